@@ -47,6 +47,7 @@ def cpu_ops(monkeypatch):
                  "prefill_attention_tile_tokens", "paged_attention_prefill", "linear_partials", "linear_partials_pay", "linear_rope_cache_write",
                  "scaled_add_rmsnorm", "mlstm_scan", "gated_head_norm", "latent_tile_tokens", "latent_attention_mfma_fits", "latent_prepare", "rotate_pairs",
                  "latent_attention", "heads_linear", "experts_linear", "route", "combine", "activation", "compute_units",
-                 "streams_norm", "delta_prepare", "delta_scan", "kv_cache_write", "local_attention", "local_attention_mfma_fits"):
+                 "streams_norm", "delta_prepare", "delta_scan", "kv_cache_write", "local_attention", "local_attention_mfma_fits",
+                 "pool_blocks", "head_norm_rotate", "decay_scan", "silu_float", "bigram_embedding", "sandwich_norm", "normed_sum"):
         monkeypatch.setattr(ops, name, getattr(emulated_ops, name))
     return ops

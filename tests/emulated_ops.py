@@ -326,7 +326,7 @@ def local_attention_mfma_fits(dtype, dim, vdim, page_size):
 
 
 def local_attention(q, out, k_plane, v_plane, block_table, token_req, positions, heads, kv_heads, dim, vdim, page_size, scale,
-                    softcap=0.0, chunk=0, window=0, gain=1.0, tiles=None):
+                    softcap=0.0, chunk=0, window=0, gain=1.0, tiles=None, sink=None, pooled=None):
     group = heads // kv_heads
     for t in range(q.shape[0]):
         p, r = int(positions[t]), int(token_req[t])
@@ -339,15 +339,119 @@ def local_attention(q, out, k_plane, v_plane, block_table, token_req, positions,
         pages = block_table[r, keys // page_size].long()
         k = k_plane[pages, :, keys % page_size].float().repeat_interleave(group, dim=1)      # [n, heads, dim]
         v = v_plane[pages, :, :, keys % page_size].float().repeat_interleave(group, dim=1)
+        if pooled is not None:
+            pk_plane, pv_plane, pool_table, pool = pooled
+            rows = torch.arange(max(0, p - window + 1) // pool)
+            ppages = pool_table[r, rows // page_size].long()
+            k = torch.cat((pk_plane[ppages, :, rows % page_size].float().repeat_interleave(group, dim=1), k))
+            v = torch.cat((pv_plane[ppages, :, :, rows % page_size].float().repeat_interleave(group, dim=1), v))
         s = torch.einsum("hd,nhd->hn", q[t].float().view(heads, dim), k) * scale
         if softcap:
             s = softcap * torch.tanh(s / softcap)
-        out[t] = (torch.einsum("hn,nhd->hd", torch.softmax(s, -1), v).reshape(-1) * gain).to(out.dtype)
+        if sink is not None:
+            w = torch.softmax(torch.cat((s, sink.float()[:, None]), -1), -1)[:, :-1]
+        else:
+            w = torch.softmax(s, -1)
+        out[t] = (torch.einsum("hn,nhd->hd", w, v).reshape(-1) * gain).to(out.dtype)
+
+
+def pool_blocks(k_plane, v_plane, block_table, pk_plane, pv_plane, pool_table, req_indptr, ctx_lens, most_blocks, page_size, pool):
+    for r in range(req_indptr.numel() - 1):
+        ctx, n = int(ctx_lens[r]), int(req_indptr[r + 1]) - int(req_indptr[r])
+        assert (ctx + n) // pool - ctx // pool <= most_blocks
+        for b in range(ctx // pool, (ctx + n) // pool):
+            ppage = int(pool_table[r, b // page_size])
+            if not ppage:
+                continue
+            keys = torch.arange(b * pool, b * pool + pool)
+            pages = block_table[r, keys // page_size].long()
+            pk_plane[ppage, :, b % page_size] = k_plane[pages, :, keys % page_size].float().mean(0).to(pk_plane.dtype)
+            pv_plane[ppage, :, :, b % page_size] = v_plane[pages, :, :, keys % page_size].float().mean(0).to(pv_plane.dtype)
+
+
+def head_norm_rotate(x, heads_a, heads_b, dim, norm_a, norm_b, eps, positions, inv_freq, dims, halves):
+    T = x.shape[0]
+    v = x.float().reshape(T, heads_a + heads_b, dim).clone()
+    if norm_a is not None or norm_b is not None:
+        w = torch.cat([(norm_a if norm_a is not None else torch.ones(dim)).float().expand(heads_a, dim),
+                       (norm_b if norm_b is not None else torch.ones(dim)).float().expand(heads_b, dim)])
+        v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w
+    if inv_freq is not None:
+        ang = positions.float()[:, None, None] * inv_freq.float()[None, None, :]
+        c, sn = ang.cos(), ang.sin()
+        if halves:
+            a, b = v[..., : dims // 2].clone(), v[..., dims // 2: dims].clone()
+            v[..., : dims // 2], v[..., dims // 2: dims] = a * c - b * sn, b * c + a * sn
+        else:
+            a, b = v[..., 0:dims:2].clone(), v[..., 1:dims:2].clone()
+            v[..., 0:dims:2], v[..., 1:dims:2] = a * c - b * sn, b * c + a * sn
+    x.copy_(v.reshape(T, -1).to(x.dtype))
+
+
+def decay_scan(qkv, decay, state, slots, req_indptr, out, heads, dim, vdim, max_new_tokens=None):
+    for r in range(req_indptr.numel() - 1):
+        st = state[int(slots[r])]
+        S = st[: heads * dim * vdim].view(heads, vdim, dim).transpose(1, 2).clone()
+        for t in range(int(req_indptr[r]), int(req_indptr[r + 1])):
+            q = qkv[t, : heads * dim].view(heads, dim)
+            k = qkv[t, heads * dim: 2 * heads * dim].view(heads, dim)
+            v = qkv[t, 2 * heads * dim:].view(heads, vdim)
+            S = S * decay[:, None, None] + k[:, :, None] * v[:, None, :]
+            out[t] = torch.einsum("hde,hd->he", S, q).reshape(-1)
+        st[: heads * dim * vdim] = S.transpose(1, 2).reshape(-1)
+
+
+def silu_float(x, out):
+    v = x.float()
+    out.copy_(v * torch.sigmoid(v))
+
+
+def bigram_embedding(token_ids, table, out, scale, bigram, buckets, mul_prev, mul_cur, token_req, req_indptr, positions, slots, last_token):
+    rows = []
+    for t in range(token_ids.numel()):
+        r = int(token_req[t])
+        if int(positions[t]) == 0:
+            rows.append(buckets)
+        else:
+            prev = int(token_ids[t - 1]) if t > int(req_indptr[r]) else int(last_token[int(slots[r]), 0])
+            rows.append((prev * mul_prev + int(token_ids[t]) * mul_cur) % buckets)
+    x = table.float()[token_ids.long()] * scale + bigram.float()[torch.tensor(rows, dtype=torch.long)]
+    out.copy_(x if out.dim() == 2 else x[None].expand_as(out))
+    for r in range(req_indptr.numel() - 1):
+        if int(req_indptr[r + 1]) > int(req_indptr[r]):
+            last_token[int(slots[r]), 0] = int(token_ids[int(req_indptr[r + 1]) - 1])
+
+
+def sandwich_norm(residual, pending, post_weight, post_eps, extra, weight, eps, out, rows=None, gain=1.0):
+    y = None
+    if pending is not None:
+        y = pending.sum(0) if pending.dim() == 3 else pending.float()
+        if post_weight is not None:
+            y = y / torch.sqrt(y.pow(2).mean(-1, keepdim=True) + post_eps) * post_weight.float()
+    r = residual if rows is None else residual[rows.long()]
+    add = None
+    if extra is not None:
+        add = extra if rows is None else extra[rows.long()]
+    if y is not None:
+        y = y if rows is None else y[rows.long()]
+        add = y if add is None else add + y
+    if add is not None:
+        if rows is None:
+            residual += add
+            r = residual
+        else:
+            r = r + add
+    out.copy_((r / torch.sqrt(r.pow(2).mean(-1, keepdim=True) + eps) * gain * weight.float()).to(out.dtype))
+
+
+def normed_sum(x, weights, eps, out):
+    v = x.float()
+    out.copy_((v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * weights[:, None, :]).sum(0).to(out.dtype))
 
 
 LATENT_ATTENTION_ROWS = 16
 LATENT_MAX_RANK = 1024
-ACTIVATIONS = {"none": 0, "relu2": 1, "silu": 2, "gelu_tanh": 3, "relu2_pairs": 17, "silu_pairs": 18, "gelu_tanh_pairs": 19}
+ACTIVATIONS = {"none": 0, "relu2": 1, "silu": 2, "gelu_tanh": 3, "gelu": 4, "relu2_pairs": 17, "silu_pairs": 18, "gelu_tanh_pairs": 19, "gelu_pairs": 20}
 
 
 LATENT_MFMA_ROWS = 64
@@ -438,6 +542,8 @@ def _act(y, activation):
         return y * torch.sigmoid(y)
     if activation == "gelu_tanh":
         return 0.5 * y * (1 + torch.tanh(math.sqrt(2 / math.pi) * (y + 0.044715 * y ** 3)))
+    if activation == "gelu":
+        return 0.5 * y * (1 + torch.erf(y / math.sqrt(2.0)))
     return y
 
 

@@ -90,6 +90,7 @@ class LayerCache:
     page_size: int
     state: torch.Tensor | None        # [slots, *shape] of the run's StateNeed
     writable: bool                    # False: the run reads another run's cache
+    more: tuple = ()                  # a mixer with several paged needs: (group, planes) of the second, third, ...
 
 
 class _PageTable:
@@ -136,6 +137,7 @@ class _PageTable:
 class _Group:
     def __init__(self, need: PagedNeed, num_pages: int):
         self.need = need
+        self.span = 1                             # positions that one page covers: page_size * need.stride
         self.runs: list[int] = []                 # indices into the run order, in order
         self.pool = PagePool(num_pages)
         self.tables: dict[object, _PageTable] = {}  # request -> page of each logical block (0: none)
@@ -172,6 +174,7 @@ class CacheManager:
         self.groups: list[_Group] = []
         self._run_group: list[int | None] = []
         self._run_index: list[int] = []          # index of the run inside its group's tensor
+        self._run_more: list[tuple] = []         # (group, index) of a run's further paged needs
         self._run_owner: list[int] = []          # run whose cache this run uses
         self._state_needs: list[StateNeed | None] = []
         self._states: list[torch.Tensor | None] = []
@@ -182,19 +185,24 @@ class CacheManager:
             if cache_of is not None:
                 self._run_group.append(self._run_group[owner])
                 self._run_index.append(self._run_index[owner])
+                self._run_more.append(self._run_more[owner])
                 self._state_needs.append(None)
                 continue
-            if paged is None:
-                self._run_group.append(None)
-                self._run_index.append(-1)
-            else:
-                g = by_need.get(paged)
+            needs = () if paged is None else (paged,) if isinstance(paged, PagedNeed) else tuple(paged)
+            placed = []
+            for need in needs:
+                if need.stride < 1:
+                    raise ValueError(f"a paged need's stride must be at least 1, got {need.stride}")
+                g = by_need.get(need)
                 if g is None:
-                    g = by_need[paged] = len(self.groups)
-                    self.groups.append(_Group(paged, self._pool_size(paged)))
-                self._run_group.append(g)
-                self._run_index.append(len(self.groups[g].runs))
+                    g = by_need[need] = len(self.groups)
+                    self.groups.append(_Group(need, self._pool_size(need)))
+                    self.groups[g].span = page_size * need.stride
+                placed.append((g, len(self.groups[g].runs)))
                 self.groups[g].runs.append(i)
+            self._run_group.append(placed[0][0] if placed else None)
+            self._run_index.append(placed[0][1] if placed else -1)
+            self._run_more.append(tuple(placed[1:]))
             self._state_needs.append(state)
         self._requests: dict[object, _Request] = {}
         self._free_slots = list(range(max_requests - 1, -1, -1))
@@ -215,13 +223,18 @@ class CacheManager:
         one the step writes.  ``None``: no bound (no window, or steps of any size)."""
         if not need.bounded or self.max_step_tokens is None:
             return None
-        return (need.reach + self.max_step_tokens - 2) // self.page_size + 2
+        return (need.reach + self.max_step_tokens - 2) // (self.page_size * need.stride) + 2
 
     def _pool_size(self, need: PagedNeed) -> int:
+        pages = self.num_pages
+        if need.stride > 1:
+            # a page spans `stride` times as many positions: as many pages as the tokens of the plain pool fill, and one more for every
+            # request, whose last page is begun however few tokens it holds
+            pages = -(-(self.num_pages - 1) // need.stride) + self.max_requests + 1
         most = self._held_at_most(need)
         if most is None:
-            return self.num_pages
-        return max(2, min(self.num_pages, self.max_requests * most + 1))
+            return pages
+        return max(2, min(pages, self.max_requests * most + 1))
 
     # ------------------------------------------------------------------ queries
     def bytes_per_page(self) -> int:
@@ -231,7 +244,8 @@ class CacheManager:
             if self._held_at_most(g.need) is not None and g.pool.num_pages < self.num_pages:
                 continue
             size = torch.empty((), dtype=g.need.dtype or self.dtype).element_size()
-            total += sum(len(g.runs) * heads * self.page_size * width * size for heads, width in g.need.plane_shapes)
+            # (a group whose rows stand for `stride` positions each grows by a page for every `stride` pages of the plain pool)
+            total += sum(len(g.runs) * heads * self.page_size * width * size for heads, width in g.need.plane_shapes) // g.need.stride
         return total
 
     def capacity(self) -> list[int]:
@@ -269,16 +283,16 @@ class CacheManager:
             first = max(first, length - g.need.window + 1)
         if g.need.chunk is not None:          # the chunk that position `length` lies in starts here; later ones start later
             first = max(first, length // g.need.chunk * g.need.chunk)
-        return first // self.page_size
+        return first // g.span
 
     def pages_missing(self, req_id, new_length: int) -> list[int]:
         """Per group, the pages that ``reserve(req_id, new_length)`` would take.  (A request's
         table holds pages exactly from the first block a query at its length can still read to
         the table's end: what is missing is counted, not looked for.)"""
         length = self._requests[req_id].length if req_id in self._requests else 0
-        blocks = -(-new_length // self.page_size)
         out = []
         for g in self.groups:
+            blocks = -(-new_length // g.span)
             held_to = len(g.tables.get(req_id, ()))
             first = self._first_live_block(g, length)
             out.append(max(0, blocks - max(first, held_to)))
@@ -288,7 +302,7 @@ class CacheManager:
         """Per group, the most pages a request holds at once on its way to ``length`` tokens."""
         out = []
         for g in self.groups:
-            blocks = -(-length // self.page_size)
+            blocks = -(-length // g.span)
             most = self._held_at_most(g.need)
             out.append(blocks if most is None else min(blocks, most))
         return out
@@ -317,8 +331,8 @@ class CacheManager:
         missing = self.pages_missing(req_id, new_length)
         if any(m > g.pool.free for m, g in zip(missing, self.groups)):
             return False
-        blocks = -(-new_length // self.page_size)
         for g in self.groups:
+            blocks = -(-new_length // g.span)
             table = g.tables[req_id]
             first = self._first_live_block(g, r.length)
             if len(table) < min(first, blocks):         # blocks no query of the step can read: never held
@@ -383,7 +397,8 @@ class CacheManager:
         planes: tuple = ()
         if gi is not None:
             planes = tuple(t[self._run_index[owner]] for t in self.groups[gi].tensors)
-        return LayerCache(group=gi, planes=planes, page_size=self.page_size, state=state, writable=(owner == run))
+        more = tuple((g, tuple(t[index] for t in self.groups[g].tensors)) for g, index in self._run_more[owner])
+        return LayerCache(group=gi, planes=planes, page_size=self.page_size, state=state, writable=(owner == run), more=more)
 
     def check(self) -> None:
         """Invariant: every page of a group is either free or held by exactly one request."""

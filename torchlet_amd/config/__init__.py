@@ -1,11 +1,13 @@
-from .base import (AttentionSpec, BlockSpec, CappedAttentionSpec, ConfigError, DenseFFSpec, GatedDeltaSpec, HyperBlockSpec, LatentAttentionSpec,
+from .base import (AttentionSpec, BlockSpec, CappedAttentionSpec, ConfigError, DecayedLinearSpec, DenseFFSpec, GatedDeltaSpec, HalfRotarySpec,
+                   HashedBigramSpec, HyperBlockSpec, LatentAttentionSpec, SandwichBlockSpec, ScalarRMSNormSpec,
                    LayerNormSpec, MLSTMSpec, ModelConfig, ModelSpec, PairRotarySpec, ParallelMixerSpec, PartSpec, PostNormBlockSpec, RMSNormSpec,
                    RotarySpec, RoutedExpertsSpec, RunEntry, SwiGLUSpec)
+from .fotovik import FotovikConfig
 from .migurax import MiguraxConfig
 from .nebutar import NebutarConfig
 from .qwen2 import Qwen2Config
 
-__all__ = ["AttentionSpec", "BlockSpec", "CappedAttentionSpec", "ConfigError", "DenseFFSpec", "GatedDeltaSpec", "HyperBlockSpec",
+__all__ = ["DecayedLinearSpec", "HalfRotarySpec", "HashedBigramSpec", "SandwichBlockSpec", "ScalarRMSNormSpec", "AttentionSpec", "BlockSpec", "CappedAttentionSpec", "ConfigError", "DenseFFSpec", "GatedDeltaSpec", "HyperBlockSpec",
            "LatentAttentionSpec", "LayerNormSpec", "MLSTMSpec", "ModelConfig", "ModelSpec", "PairRotarySpec", "ParallelMixerSpec", "PartSpec",
-           "PostNormBlockSpec", "RMSNormSpec", "RotarySpec", "RoutedExpertsSpec", "RunEntry", "SwiGLUSpec", "MiguraxConfig", "NebutarConfig",
+           "PostNormBlockSpec", "RMSNormSpec", "RotarySpec", "RoutedExpertsSpec", "RunEntry", "SwiGLUSpec", "FotovikConfig", "MiguraxConfig", "NebutarConfig",
            "Qwen2Config"]

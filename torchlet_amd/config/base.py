@@ -48,6 +48,16 @@ class LayerNormSpec(PartSpec):
 
 
 @dataclass(frozen=True)
+class ScalarRMSNormSpec(PartSpec):
+    """``x / sqrt(mean(x^2) + eps) * g`` with one number ``g`` for all coordinates (a tensor without axes).  ``weight_name`` as in
+    :class:`RMSNormSpec`."""
+    kind: ClassVar[str] = "scalar_rmsnorm"
+    dim: int = 0
+    eps: float = 1e-6
+    weight_name: str = "weight"
+
+
+@dataclass(frozen=True)
 class RotarySpec(PartSpec):
     """Split-half rotary position encoding over the whole head."""
     kind: ClassVar[str] = "rope_split_half"
@@ -84,6 +94,17 @@ class PairRotarySpec(PartSpec):
     kind: ClassVar[str] = "rope_pairs"
     dims: int = 0
     base: float = 10000.0
+    factor: float = 1.0        # linear scaling: every frequency is divided by it
+
+
+@dataclass(frozen=True)
+class HalfRotarySpec(PartSpec):
+    """Rotary position encoding in the rotate-half layout over the first ``dims`` entries of a vector: entry ``i`` is paired with
+    ``i + dims / 2`` and turned by ``position * base**(-2i / dims) / factor``; what lies beyond ``dims`` passes unchanged."""
+    kind: ClassVar[str] = "rope_halves"
+    dims: int = 0
+    base: float = 10000.0
+    factor: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -138,6 +159,31 @@ class CappedAttentionSpec(PartSpec):
     softcap: float | None = None
     chunk: int | None = None
     window: int | None = None
+    # Further mechanisms, each off unless named.  ``position``: a position encoding whose ``turn`` the mixer applies to queries and keys
+    # (``rope_pairs`` or ``rope_halves``, over the first dimensions of every head).  ``qk_norm``: queries and keys pass a root-mean-square norm
+    # per head before the rotation, with the weights ``q.norm`` and ``k.norm`` of ``dim`` numbers each, shared by all heads (``qk_norm_eps``).
+    # ``sink``: the softmax's denominator also holds ``exp`` of one learned number per head (tensor ``sink``), unscaled, without key or
+    # value.  ``pool``: with a window, one key and one value (the means of the cached ones) for every block of ``pool`` positions that lies
+    # wholly before the window; tokens that have left the window and whose block is not whole yet are not read at all.
+    position: PartSpec | None = None
+    qk_norm: bool = False
+    qk_norm_eps: float = 1e-6
+    sink: bool = False
+    pool: int | None = None
+
+
+@dataclass(frozen=True)
+class DecayedLinearSpec(PartSpec):
+    """Linear attention with one fixed decay per head (lightning attention): ``q = silu(W_q h)``, ``k = silu(W_k h)`` (``heads x dim``),
+    ``v = silu(W_v h)`` (``heads x vdim``); per head ``S <- decay S + k v^T``, ``o = S^T q``; the heads side by side are divided by their
+    root mean square together (``norm_eps``), multiplied by a weight vector and by ``sigmoid(W_g h)``, and projected."""
+    kind: ClassVar[str] = "decayed_linear"
+    hidden: int = 0
+    heads: int = 0
+    dim: int = 0
+    vdim: int = 0
+    decay: tuple = ()
+    norm_eps: float = 1e-6
 
 
 @dataclass(frozen=True)
@@ -166,6 +212,10 @@ class ParallelMixerSpec(PartSpec):
     kind: ClassVar[str] = "parallel"
     hidden: int = 0
     branches: tuple = ()
+    # ``normed``: every branch's projected output is first divided by its root mean square over the model width (``norm_eps``) and
+    # multiplied by a weight vector ``<name>.out``: ``sum_i scale_i * rms(mixer_i(h)) * w_i``.
+    normed: bool = False
+    norm_eps: float = 1e-6
 
 
 @dataclass(frozen=True)
@@ -225,6 +275,17 @@ class PostNormBlockSpec(BlockSpec):
 
 
 @dataclass(frozen=True)
+class SandwichBlockSpec(BlockSpec):
+    """One layer with a norm before and after each sublayer: ``x <- x + mixer_post_norm(mixer(mixer_norm(x)))``, then ``x <- x +
+    ffn_post_norm(ffn(ffn_norm(x)))``.  ``ffn`` (and then its two norms) may be ``None``."""
+    kind: ClassVar[str] = "sandwich_residual"
+    mixer_post_norm: PartSpec = None       # type: ignore[assignment]
+    ffn_post_norm: PartSpec = None         # type: ignore[assignment]
+    mixer_post_norm_name: str = "norm1b"
+    ffn_post_norm_name: str = "norm2b"
+
+
+@dataclass(frozen=True)
 class HyperBlockSpec(BlockSpec):
     """One layer over ``streams`` copies of the residual joined by hyper-connections.  Sublayer ``q`` (1: the mixer, 2: the
     feed-forward) has a read vector ``in [streams]``, a matrix ``mix [streams, streams]`` (indexed from, to) and a write vector
@@ -245,6 +306,17 @@ class RunEntry:
     """
     layer: int
     cache_of: int | None = None
+    add_embedding: bool = False     # the embedding's output (the stream as it was before the first run) is added to the stream before this run
+
+
+@dataclass(frozen=True)
+class HashedBigramSpec:
+    """A second embedding table ``[buckets + 1, hidden]`` under ``name`` whose row ``(previous token * mul_prev + token * mul_cur) mod
+    buckets`` is added to a token's embedding; a sequence's first token takes the last row.  The previous token is part of a request's state."""
+    name: str = "bigram"
+    buckets: int = 0
+    mul_prev: int = 0
+    mul_cur: int = 0
 
 
 @dataclass(frozen=True)
@@ -268,6 +340,7 @@ class ModelSpec:
     layers_format: str = ""        # the name of layer i as a format string (``"l{}"``); empty: ``<layers_prefix>.<i>``
     position_table_name: str = ""  # a learned table ``[max_positions, hidden]`` whose row of the position is added to the (scaled) embedding; empty: none
     streams: int = 0               # copies of the residual that the blocks keep (hyper-connections); 0: the one plain residual
+    bigram: HashedBigramSpec | None = None   # a hashed bigram row added to every token's (scaled) embedding
 
     def layer_name(self, i: int) -> str:
         return self.layers_format.format(i) if self.layers_format else f"{self.layers_prefix}.{i}"

@@ -677,3 +677,163 @@ extern "C" int tl_streams_norm(void* x, int streams, int total_rows, int hidden,
     TL_CHECK_LAUNCH("streams_norm");
     return TL_OK;
 }
+
+// ------------------------------------------------------------------ embedding with a hashed bigram row
+// out[c, t, :] = float(table[ids[t], :]) * scale + float(bigram[row(t), :]), row(t) = (prev * mul_prev + ids[t] * mul_cur) mod buckets with prev
+// the token before t in its sequence, or row `buckets` (the table's last) for a sequence's first token (position 0).  The token before a
+// step's first token of a request is read from last_token[slot] (what the step before left there); last_token_kernel moves it on.
+template <typename T>
+__global__ void bigram_embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int hidden, int vocab,
+                                        float scale, const int* __restrict__ token_req, const int* __restrict__ req_indptr,
+                                        const int* __restrict__ positions, const int* __restrict__ slots, const int* __restrict__ last_token,
+                                        const T* __restrict__ bigram, int buckets, long long mul_prev, long long mul_cur, int copies, size_t copy_stride) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    if (id < 0 || id >= vocab) id = 0;
+    const int r = token_req[t];
+    int row = buckets;
+    if (positions[t] > 0) {
+        int prev = t > req_indptr[r] ? ids[t - 1] : last_token[slots[r]];
+        if (prev < 0 || prev >= vocab) prev = 0;
+        long long h = ((long long)prev * mul_prev + (long long)id * mul_cur) % buckets;
+        if (h < 0) h += buckets;
+        row = (int)h;
+    }
+    const T* src = table + (size_t)id * hidden;
+    const T* big = bigram + (size_t)row * hidden;
+    float* dst = out + (size_t)t * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float v = fmaf(to_float(src[i]), scale, to_float(big[i]));
+        for (int c = 0; c < copies; ++c) dst[c * copy_stride + i] = v;
+    }
+}
+
+__global__ void last_token_kernel(const int* __restrict__ ids, const int* __restrict__ req_indptr, const int* __restrict__ slots,
+                                  int* __restrict__ last_token, int requests) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= requests) return;
+    const int a = req_indptr[r], b = req_indptr[r + 1];
+    if (b > a) last_token[slots[r]] = ids[b - 1];
+}
+
+extern "C" int tl_bigram_embedding(const void* ids, const void* table, void* out, int tokens, int hidden, int vocab, float scale,
+                                   const void* token_req, const void* req_indptr, int requests, const void* positions, const void* slots,
+                                   void* last_token, const void* bigram, int buckets, long mul_prev, long mul_cur, int copies, int dtype,
+                                   hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0 && copies > 0 && buckets > 0 && requests >= 0, "bigram_embedding: bad sizes");
+    TL_REQUIRE(token_req && req_indptr && positions && slots && last_token && bigram, "bigram_embedding: a null operand");
+    if (tokens == 0) return TL_OK;
+    const size_t copy_stride = (size_t)tokens * hidden;
+    if (dtype == TL_DT_F32)
+        bigram_embedding_kernel<float><<<tokens, 256, 0, stream>>>((const int*)ids, (const float*)table, (float*)out, hidden, vocab, scale,
+            (const int*)token_req, (const int*)req_indptr, (const int*)positions, (const int*)slots, (const int*)last_token, (const float*)bigram,
+            buckets, mul_prev, mul_cur, copies, copy_stride);
+    else if (dtype == TL_DT_BF16)
+        bigram_embedding_kernel<bf16_t><<<tokens, 256, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab, scale,
+            (const int*)token_req, (const int*)req_indptr, (const int*)positions, (const int*)slots, (const int*)last_token, (const bf16_t*)bigram,
+            buckets, mul_prev, mul_cur, copies, copy_stride);
+    else TL_REQUIRE(false, "bigram_embedding: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("bigram_embedding");
+    last_token_kernel<<<(requests + 63) / 64, 64, 0, stream>>>((const int*)ids, (const int*)req_indptr, (const int*)slots, (int*)last_token, requests);
+    TL_CHECK_LAUNCH("last_token");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ norm of the branch output, addition, norm of the sum
+// One block per output row, the row kept in shared memory between the passes:
+//   y = pending[row] (one tensor of the activation type, or `parts` float slabs added up);
+//   r = residual[row] (+ extra[row]) + y * (post ? rsqrt(mean(y^2) + post_eps) * post[i] : 1);   written back unless `rows` selects
+//   out = r * rsqrt(mean(r^2) + eps) * weight[i] * gain.
+// `post` and `weight` are float vectors of post_n / weight_n numbers: `hidden` of them, or one for all coordinates.
+template <typename T>
+__global__ void sandwich_norm_kernel(float* __restrict__ residual, const void* __restrict__ pending, int parts, size_t part_stride,
+                                     const float* __restrict__ post, int post_n, float post_eps, const float* __restrict__ extra,
+                                     const float* __restrict__ weight, int weight_n, float eps, float gain, T* __restrict__ out,
+                                     const int* __restrict__ rows, int hidden) {
+    extern __shared__ float sn_row[];
+    __shared__ float red[16];
+    const int orow = blockIdx.x;
+    const int srow = rows ? rows[orow] : orow;
+    float* res = residual + (size_t)srow * hidden;
+    const T* pen = (pending && parts == 0) ? (const T*)pending + (size_t)srow * hidden : nullptr;
+    const float* pparts = (pending && parts > 0) ? (const float*)pending + (size_t)srow * hidden : nullptr;
+    const float* ex = extra ? extra + (size_t)srow * hidden : nullptr;
+    float inv_y = 1.f;
+    if (pending) {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+            float y = 0.f;
+            if (pen) y = to_float(pen[i]);
+            if (pparts)
+                for (int p = 0; p < parts; ++p) y += pparts[p * part_stride + i];
+            sn_row[i] = y;
+            ss = fmaf(y, y, ss);
+        }
+        if (post) inv_y = rsqrtf(block_sum(ss, red) / (float)hidden + post_eps);
+    }
+    const bool update = (pending != nullptr || ex != nullptr) && rows == nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float r = res[i];
+        if (ex) r += ex[i];
+        if (pending) r += post ? sn_row[i] * inv_y * post[post_n == 1 ? 0 : i] : sn_row[i];
+        if (update) res[i] = r;
+        sn_row[i] = r;
+        ss = fmaf(r, r, ss);
+    }
+    const float inv = rsqrtf(block_sum(ss, red) / (float)hidden + eps) * gain;
+    T* dst = out + (size_t)orow * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = from_float<T>(sn_row[i] * inv * weight[weight_n == 1 ? 0 : i]);
+}
+
+extern "C" int tl_sandwich_norm(void* residual, const void* pending, int parts, int part_rows, const void* post, int post_n, float post_eps,
+                                const void* extra, const void* weight, int weight_n, float eps, float gain, void* out, const void* rows,
+                                int out_rows, int hidden, int act_dtype, hipStream_t stream) {
+    TL_REQUIRE(parts >= 0 && parts <= 64 && out_rows >= 0 && hidden > 0 && hidden <= 12288, "sandwich_norm: bad sizes rows=%d hidden=%d parts=%d", out_rows, hidden, parts);
+    TL_REQUIRE(weight && (weight_n == 1 || weight_n == hidden) && (!post || post_n == 1 || post_n == hidden), "sandwich_norm: weights of one number or of %d", hidden);
+    if (out_rows == 0) return TL_OK;
+    const size_t part_stride = (size_t)part_rows * hidden, smem = sizeof(float) * hidden;
+    const int threads = hidden >= 2048 ? 512 : 256;
+    if (act_dtype == TL_DT_F32)
+        sandwich_norm_kernel<float><<<out_rows, threads, smem, stream>>>((float*)residual, pending, parts, part_stride, (const float*)post, post_n, post_eps,
+            (const float*)extra, (const float*)weight, weight_n, eps, gain, (float*)out, (const int*)rows, hidden);
+    else if (act_dtype == TL_DT_BF16)
+        sandwich_norm_kernel<bf16_t><<<out_rows, threads, smem, stream>>>((float*)residual, pending, parts, part_stride, (const float*)post, post_n, post_eps,
+            (const float*)extra, (const float*)weight, weight_n, eps, gain, (bf16_t*)out, (const int*)rows, hidden);
+    else TL_REQUIRE(false, "sandwich_norm: unknown dtype %d", act_dtype);
+    TL_CHECK_LAUNCH("sandwich_norm");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ sum of normed branches
+// out[t, :] = sum_b x[b, t, :] * rsqrt(mean(x[b, t, :]^2) + eps) * w[b, :] over `branches` tensors side by side; one block per row, float sums.
+#define NS_MAX_BRANCHES 8
+template <typename T>
+__global__ void normed_sum_kernel(const T* __restrict__ x, int branches, size_t branch_stride, const float* __restrict__ w, float eps,
+                                  T* __restrict__ out, int hidden) {
+    __shared__ float red[16];
+    const int row = blockIdx.x;
+    float inv[NS_MAX_BRANCHES];
+    for (int b = 0; b < branches; ++b) {
+        const T* src = x + b * branch_stride + (size_t)row * hidden;
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < hidden; i += blockDim.x) { const float v = to_float(src[i]); ss = fmaf(v, v, ss); }
+        inv[b] = rsqrtf(block_sum(ss, red) / (float)hidden + eps);
+    }
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float y = 0.f;
+        for (int b = 0; b < branches; ++b) y = fmaf(to_float(x[b * branch_stride + (size_t)row * hidden + i]) * inv[b], w[(size_t)b * hidden + i], y);
+        out[(size_t)row * hidden + i] = from_float<T>(y);
+    }
+}
+
+extern "C" int tl_normed_sum(const void* x, int branches, int rows, int hidden, const void* w, float eps, void* out, int dtype, hipStream_t stream) {
+    TL_REQUIRE(branches > 0 && branches <= NS_MAX_BRANCHES && rows >= 0 && hidden > 0, "normed_sum: bad sizes (up to %d branches)", NS_MAX_BRANCHES);
+    if (rows == 0) return TL_OK;
+    const size_t stride = (size_t)rows * hidden;
+    if (dtype == TL_DT_F32) normed_sum_kernel<float><<<rows, 256, 0, stream>>>((const float*)x, branches, stride, (const float*)w, eps, (float*)out, hidden);
+    else if (dtype == TL_DT_BF16) normed_sum_kernel<bf16_t><<<rows, 256, 0, stream>>>((const bf16_t*)x, branches, stride, (const float*)w, eps, (bf16_t*)out, hidden);
+    else TL_REQUIRE(false, "normed_sum: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("normed_sum");
+    return TL_OK;
+}

@@ -7,16 +7,18 @@
 #define ACT_RELU2 1
 #define ACT_SILU 2
 #define ACT_GELU_TANH 3
+#define ACT_GELU 4        // the exact form, with the error function
 #define ACT_PAIRS 16      // added to one of the above: the product's columns 2i and 2i + 1 are a gate and an up value, the output act(gate) * up
 
 __device__ __forceinline__ float activate(float v, int act) {
     if (act == ACT_RELU2) { v = fmaxf(v, 0.f); return v * v; }
     if (act == ACT_SILU) return v / (1.f + expf(-v));
     if (act == ACT_GELU_TANH) return 0.5f * v * (1.f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    if (act == ACT_GELU) return 0.5f * v * (1.f + erff(v * 0.7071067811865476f));
     return v;
 }
 
-__host__ __device__ __forceinline__ bool known_activation(int act) { return (act & ~ACT_PAIRS) >= ACT_NONE && (act & ~ACT_PAIRS) <= ACT_GELU_TANH; }
+__host__ __device__ __forceinline__ bool known_activation(int act) { return (act & ~ACT_PAIRS) >= ACT_NONE && (act & ~ACT_PAIRS) <= ACT_GELU; }
 
 // ------------------------------------------------------------------ grouped product
 // out[row(m), g_out + n] = act(sum_k a[src(m), g_a + k] * w[g][n][k]) for the rows m of group g, in tiles of 64 x 64

@@ -4,6 +4,11 @@
 //   k_plane [pages, kv_heads, page_size, dim], v_plane [pages, kv_heads, vdim, page_size] (the values of a page lie transposed, so
 //   that eight neighbouring keys' values of one column are 16 bytes side by side, which is how the matrix cores want them); key j
 //   of a request lies in slot j % page_size of page block_table[request][j / page_size].
+// Two more mechanisms, each switched on by its operand.  A sink: the softmax's denominator also holds exp(sink[head]), which has neither
+// key nor value and is not scaled.  Pooled blocks: beside a window of `window` tokens a query at position p reads one key and one
+// value for every block of `pool` positions that lies wholly before its window, blocks 0 .. (p - window + 1) / pool - 1; block b's key
+// and value are the means of the cached keys and values of the positions b * pool .. b * pool + pool - 1 and lie, as a token's would, in
+// row b of planes of their own with a block table of their own (pool_blocks_kernel makes them when a step brings a block's last token).
 #include "common.h"
 
 // ------------------------------------------------------------------ cache write
@@ -74,7 +79,8 @@ __global__ void __launch_bounds__(LA_WAVES * TL_WAVE)
 local_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, int out_ld, const T* __restrict__ k_plane,
                        const T* __restrict__ v_plane, const int* __restrict__ block_table, int table_ld, const int* __restrict__ token_req,
                        const int* __restrict__ positions, int heads, int kv_heads, int dim, int vdim, int page_size, float scale, float cap,
-                       LocalMask mask, float gain) {
+                       LocalMask mask, float gain, const float* __restrict__ sink, const T* __restrict__ pk_plane, const T* __restrict__ pv_plane,
+                       const int* __restrict__ pool_table, int pool_table_ld, int pool) {
     __shared__ float sq[LA_MAX_DIM];
     __shared__ float sm[LA_WAVES], sl[LA_WAVES];
     __shared__ float sacc[LA_WAVES][LA_MAX_DIM];
@@ -84,6 +90,8 @@ local_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, i
     const int p = positions[t];
     const int lo = mask.first(p);
     const int* table = block_table + (size_t)token_req[t] * table_ld;
+    const int* ptable = pool > 0 ? pool_table + (size_t)token_req[t] * pool_table_ld : nullptr;
+    const int npool = (pool > 0 && mask.window > 0) ? max(0, p - mask.window + 1) / pool : 0;      // pooled blocks: keys 0 .. npool - 1 of this query
     for (int d = threadIdx.x; d < dim; d += blockDim.x) sq[d] = to_float(q[(size_t)t * q_ld + head * dim + d]) * scale;
     __syncthreads();
 
@@ -91,18 +99,20 @@ local_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, i
     float acc[LA_COLS];
 #pragma unroll
     for (int c = 0; c < LA_COLS; ++c) acc[c] = 0.f;
-    const int nkeys = p - lo + 1;
+    const int nkeys = npool + p - lo + 1;
     for (int b = wave; b * TL_WAVE < nkeys; b += LA_WAVES) {
-        const int j = lo + b * TL_WAVE + lane;
-        const bool ok = j <= p;
+        const int u = b * TL_WAVE + lane;                // pooled blocks first, then the tokens lo .. p
+        const bool ok = u < nkeys;
         float s = -INFINITY;
-        size_t at = 0;                                 // page and head of the key, and its slot
-        int slot = 0;
+        const T* vr0 = v_plane;                          // the key's values: column c at vr0[c * page_size]
         if (ok) {
-            const int page = table[j / page_size];
-            at = (size_t)page * kv_heads + g;
-            slot = j % page_size;
-            const T* kr = k_plane + (at * page_size + slot) * dim;
+            const bool pooled = u < npool;
+            const int j = pooled ? u : lo + u - npool;
+            const int page = (pooled ? ptable : table)[j / page_size];
+            const size_t at = (size_t)page * kv_heads + g;
+            const int slot = j % page_size;
+            const T* kr = (pooled ? pk_plane : k_plane) + (at * page_size + slot) * dim;
+            vr0 = (pooled ? pv_plane : v_plane) + at * vdim * page_size + slot;
             float dot = 0.f;
             for (int d = 0; d < dim; ++d) dot = fmaf(sq[d], to_float(kr[d]), dot);
             s = cap_score(dot, cap);
@@ -114,11 +124,12 @@ local_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, i
         m = m_new;
 #pragma unroll
         for (int c = 0; c < LA_COLS; ++c) acc[c] *= keep;
-        const int nb = min(TL_WAVE, p - (lo + b * TL_WAVE) + 1);
+        const int nb = min(TL_WAVE, nkeys - b * TL_WAVE);
+        const unsigned long long vaddr = (unsigned long long)(uintptr_t)vr0;
         for (int i = 0; i < nb; ++i) {
             const float wi = __shfl(w, i, TL_WAVE);
-            const size_t ati = ((size_t)(unsigned)__shfl((int)(at >> 32), i, TL_WAVE) << 32) | (unsigned)__shfl((int)at, i, TL_WAVE);
-            const T* vr = v_plane + ati * vdim * page_size + __shfl(slot, i, TL_WAVE);
+            const unsigned long long ai = ((unsigned long long)(unsigned)__shfl((int)(vaddr >> 32), i, TL_WAVE) << 32) | (unsigned)__shfl((int)vaddr, i, TL_WAVE);
+            const T* vr = (const T*)(uintptr_t)ai;
 #pragma unroll
             for (int c = 0; c < LA_COLS; ++c) {
                 const int col = lane + c * TL_WAVE;
@@ -133,11 +144,13 @@ local_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, i
     if (wave == 0) {
         float top = sm[0];
         for (int w = 1; w < LA_WAVES; ++w) top = fmaxf(top, sm[w]);
+        if (sink) top = fmaxf(top, sink[head]);
         float den = 0.f, f[LA_WAVES];
         for (int w = 0; w < LA_WAVES; ++w) {
             f[w] = sl[w] > 0.f ? expf(sm[w] - top) : 0.f;       // a wave without keys: no share
             den = fmaf(sl[w], f[w], den);
         }
+        if (sink) den += expf(sink[head] - top);
         const float norm = gain / den;
         for (int col = lane; col < vdim; col += TL_WAVE) {
             float o = 0.f;
@@ -189,7 +202,8 @@ local_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __re
                             const bf16_t* __restrict__ v_plane, const int* __restrict__ block_table, int table_ld, int table_width,
                             const int* __restrict__ req_indptr, const int* __restrict__ ctx_lens, const int* __restrict__ tile_req,
                             const int* __restrict__ tile_tok0, int heads, int kv_heads, int page_size, float scale, float cap,
-                            LocalMask mask, float gain) {
+                            LocalMask mask, float gain, const float* __restrict__ sink, const bf16_t* __restrict__ pk_plane,
+                            const bf16_t* __restrict__ pv_plane, const int* __restrict__ pool_table, int pool_table_ld, int pool_table_width, int pool) {
     constexpr int dim = DK * 32, vdim = DV * 16;
     extern __shared__ float la_smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, kq = lane >> 4;
@@ -223,93 +237,104 @@ local_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __re
     float m = -INFINITY, l = 0.f;
 
     const int p_last = p0 + n_tile - 1;
-    const int lo_tile = mask.first(p0);                          // the first token reads furthest back; pages before may be gone
-    const int base0 = lo_tile / LAM_KEYS * LAM_KEYS;
     // rows of the two score products that this lane fetches: keys base + 8 (li / 4) + li % 4 (+ 4)
     const int krow = 8 * (li >> 2) + (li & 3);
-    // The pages of up to 64 blocks of the request lie in a register across the wave (lane i: block tab_first + i) and are read from
-    // there, so that no fetch waits for a look-up in memory; the window moves on every 64 blocks.
-    int tab_first = page_of(base0);
-    int tab_reg = table[min(tab_first + lane, table_width - 1)];
-    auto page_at = [&](int key) { return __shfl(tab_reg, page_of(key) - tab_first, TL_WAVE); };
-    // The keys and values of a step are fetched one step ahead, while the step before is worked on.
-    LaFrag a0[DK], a1[DK], va[DV], vb[DV];
-    auto fetch = [&](int base, LaFrag (&vf)[DV]) {
-        if (page_of(base + LAM_KEYS - 1) - tab_first >= TL_WAVE) {            // (the same for every lane)
-            tab_first = page_of(base);
-            tab_reg = table[min(tab_first + lane, table_width - 1)];
-        }
-        // keys: rows base + krow and base + krow + 4 (clamped into what exists: masked below)
-        const int key0 = max(min(base + krow, p_last), lo_tile), key1 = max(min(base + krow + 4, p_last), lo_tile);
-        const bf16_t* k0 = k_plane + (((size_t)page_at(key0) * kv_heads + g) * page_size + slot_of(key0)) * dim + 8 * kq;
-        const bf16_t* k1 = k_plane + (((size_t)page_at(key1) * kv_heads + g) * page_size + slot_of(key1)) * dim + 8 * kq;
+    // One pass over a stretch of keys lo_valid .. hi_valid of planes kp / vp (the tokens of the tile's reach, or the pooled blocks before its
+    // window), of which this lane's token reads my_first .. my_last.  The running maximum, sum and output carry over from pass to pass.
+    auto run = [&](const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp, const int* __restrict__ tbl, int tbl_width, int lo_valid, int hi_valid,
+                   int my_first, int my_last) {
+        const int base0 = lo_valid / LAM_KEYS * LAM_KEYS;
+        if (base0 + LAM_KEYS * wave > hi_valid) return;
+        // The pages of up to 64 blocks of the request lie in a register across the wave (lane i: block tab_first + i) and are read from
+        // there, so that no fetch waits for a look-up in memory; the window moves on every 64 blocks.
+        int tab_first = page_of(base0);
+        int tab_reg = tbl[min(tab_first + lane, tbl_width - 1)];
+        auto page_at = [&](int key) { return __shfl(tab_reg, page_of(key) - tab_first, TL_WAVE); };
+        // The keys and values of a step are fetched one step ahead, while the step before is worked on.
+        LaFrag a0[DK], a1[DK], va[DV], vb[DV];
+        auto fetch = [&](int base, LaFrag (&vf)[DV]) {
+            if (page_of(base + LAM_KEYS - 1) - tab_first >= TL_WAVE) {            // (the same for every lane)
+                tab_first = page_of(base);
+                tab_reg = tbl[min(tab_first + lane, tbl_width - 1)];
+            }
+            // keys: rows base + krow and base + krow + 4 (clamped into what exists: masked below)
+            const int key0 = max(min(base + krow, hi_valid), lo_valid), key1 = max(min(base + krow + 4, hi_valid), lo_valid);
+            const bf16_t* k0 = kp + (((size_t)page_at(key0) * kv_heads + g) * page_size + slot_of(key0)) * dim + 8 * kq;
+            const bf16_t* k1 = kp + (((size_t)page_at(key1) * kv_heads + g) * page_size + slot_of(key1)) * dim + 8 * kq;
 #pragma unroll
-        for (int s = 0; s < DK; ++s) { a0[s].u = *(const uint4*)(k0 + 32 * s); a1[s].u = *(const uint4*)(k1 + 32 * s); }
-        // values, transposed: row = column of the values, k = keys base + 8 kq .. + 7 (one page: page_size % 8 == 0)
-        const int key = base + 8 * kq;
-        const int kc = max(min(key, p_last), lo_tile);
-        const bf16_t* vt = v_plane + (((size_t)page_at(kc) * kv_heads + g) * vdim + li) * page_size + slot_of(key);
+            for (int s = 0; s < DK; ++s) { a0[s].u = *(const uint4*)(k0 + 32 * s); a1[s].u = *(const uint4*)(k1 + 32 * s); }
+            // values, transposed: row = column of the values, k = keys base + 8 kq .. + 7 (one page: page_size % 8 == 0)
+            const int key = base + 8 * kq;
+            const int kc = max(min(key, hi_valid), lo_valid);
+            const bf16_t* vt = vp + (((size_t)page_at(kc) * kv_heads + g) * vdim + li) * page_size + slot_of(key);
 #pragma unroll
-        for (int j = 0; j < DV; ++j) vf[j].u = *(const uint4*)(vt + (size_t)16 * j * page_size);      // (never conditional: nothing waits for it here)
-    };
-    auto step = [&](int base, LaFrag (&vf)[DV], LaFrag (&vnext)[DV]) {
-        // ---- scores of 32 keys
-        la_f32x4 s0 = la_f32x4{0.f, 0.f, 0.f, 0.f}, s1 = la_f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int j = 0; j < DV; ++j) vf[j].u = *(const uint4*)(vt + (size_t)16 * j * page_size);      // (never conditional: nothing waits for it here)
+        };
+        auto step = [&](int base, LaFrag (&vf)[DV], LaFrag (&vnext)[DV]) {
+            // ---- scores of 32 keys
+            la_f32x4 s0 = la_f32x4{0.f, 0.f, 0.f, 0.f}, s1 = la_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s = 0; s < DK; ++s) {
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[s].v, qf[s].v, s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[s].v, qf[s].v, s1, 0, 0, 0);
-        }
-        if (base + LAM_STRIDE <= p_last) fetch(base + LAM_STRIDE, vnext);
-        // ---- cap, mask, running maximum (scores in units of log 2 from here on, so that the weights are plain powers of two)
-        float sc[8];
-        float mx = -INFINITY;
+            for (int s = 0; s < DK; ++s) {
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[s].v, qf[s].v, s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[s].v, qf[s].v, s1, 0, 0, 0);
+            }
+            if (base + LAM_STRIDE <= hi_valid) fetch(base + LAM_STRIDE, vnext);
+            // ---- cap, mask, running maximum (scores in units of log 2 from here on, so that the weights are plain powers of two)
+            float sc[8];
+            float mx = -INFINITY;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int key = base + 8 * kq + e;
-            const float raw = (e < 4 ? s0[e] : s1[e - 4]) * scale;
-            sc[e] = (key <= my_p && key >= my_lo) ? cap_score_fast(raw, cap, inv_cap) * LA_LOG2E : -INFINITY;
-            mx = fmaxf(mx, sc[e]);
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, TL_WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, TL_WAVE));
-        const float m_new = fmaxf(m, mx);
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;   // a token that has seen no key yet
-        const float keep = __builtin_amdgcn_exp2f(m - m_use);   // (0 while m is -inf)
-        m = m_new;
-        LaFrag pf;
-        float psum = 0.f;
+            for (int e = 0; e < 8; ++e) {
+                const int key = base + 8 * kq + e;
+                const float raw = (e < 4 ? s0[e] : s1[e - 4]) * scale;
+                sc[e] = (key <= my_last && key >= my_first) ? cap_score_fast(raw, cap, inv_cap) * LA_LOG2E : -INFINITY;
+                mx = fmaxf(mx, sc[e]);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, TL_WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, TL_WAVE));
+            const float m_new = fmaxf(m, mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;   // a token that has seen no key yet
+            const float keep = __builtin_amdgcn_exp2f(m - m_use);   // (0 while m is -inf)
+            m = m_new;
+            LaFrag pf;
+            float psum = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float w = __builtin_amdgcn_exp2f(sc[e] - m_use);
-            const bf16_t wb = from_float<bf16_t>(w);
-            pf.e[e] = wb.bits;
-            psum += to_float(wb);                               // the sum of what the second product sees
-        }
-        l = l * keep + psum;
-        // places no token has written yet, or whose page is gone, may hold anything: their values count as zero (first and last steps only)
-        const int vkey = base + 8 * kq;
-        if (vkey + 7 > p_last || vkey < lo_tile) {
+            for (int e = 0; e < 8; ++e) {
+                const float w = __builtin_amdgcn_exp2f(sc[e] - m_use);
+                const bf16_t wb = from_float<bf16_t>(w);
+                pf.e[e] = wb.bits;
+                psum += to_float(wb);                               // the sum of what the second product sees
+            }
+            l = l * keep + psum;
+            // places no token has written yet, or whose page is gone, may hold anything: their values count as zero (first and last steps only)
+            const int vkey = base + 8 * kq;
+            if (vkey + 7 > hi_valid || vkey < lo_valid) {
 #pragma unroll
-            for (int j = 0; j < DV; ++j)
+                for (int j = 0; j < DV; ++j)
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (vkey + e > p_last || vkey + e < lo_tile) vf[j].e[e] = 0;
-        }
-        if (__any(keep != 1.f)) {                               // (the maxima settle after a tile's first steps)
+                    for (int e = 0; e < 8; ++e)
+                        if (vkey + e > hi_valid || vkey + e < lo_valid) vf[j].e[e] = 0;
+            }
+            if (__any(keep != 1.f)) {                               // (the maxima settle after a tile's first steps)
 #pragma unroll
-            for (int j = 0; j < DV; ++j) { acc[j][0] *= keep; acc[j][1] *= keep; acc[j][2] *= keep; acc[j][3] *= keep; }
-        }
+                for (int j = 0; j < DV; ++j) { acc[j][0] *= keep; acc[j][1] *= keep; acc[j][2] *= keep; acc[j][3] *= keep; }
+            }
 #pragma unroll
-        for (int j = 0; j < DV; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j].v, pf.v, acc[j], 0, 0, 0);
-    };
-    if (base0 + LAM_KEYS * wave <= p_last) {
+            for (int j = 0; j < DV; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j].v, pf.v, acc[j], 0, 0, 0);
+        };
         fetch(base0 + LAM_KEYS * wave, va);
-        for (int base = base0 + LAM_KEYS * wave; base <= p_last; base += 2 * LAM_STRIDE) {
+        for (int base = base0 + LAM_KEYS * wave; base <= hi_valid; base += 2 * LAM_STRIDE) {
             step(base, va, vb);
-            if (base + LAM_STRIDE <= p_last) step(base + LAM_STRIDE, vb, va);
+            if (base + LAM_STRIDE <= hi_valid) step(base + LAM_STRIDE, vb, va);
         }
+    };
+    if (pool > 0 && mask.window > 0) {
+        // the pooled blocks that lie wholly before a token's window: 0 .. (p - window + 1) / pool - 1; the tile's last token reads the most
+        const int n_tile_blocks = max(0, p_last - mask.window + 1) / pool, n_my_blocks = max(0, my_p - mask.window + 1) / pool;
+        if (n_tile_blocks > 0)
+            run(pk_plane, pv_plane, pool_table + (size_t)req * pool_table_ld, pool_table_width, 0, n_tile_blocks - 1, 0, n_my_blocks - 1);
     }
+    // the first token reads furthest back; pages before may be gone
+    run(k_plane, v_plane, table, table_width, mask.first(p0), p_last, my_lo, my_p);
     l += __shfl_xor(l, 16, TL_WAVE);
     l += __shfl_xor(l, 32, TL_WAVE);
     // ---- the four waves' shares are joined: per token the maxima, the sums and the outputs, in the order of the waves
@@ -327,7 +352,9 @@ local_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __re
         float top = sm_m[tok];
 #pragma unroll
         for (int w = 1; w < LAM_WAVES; ++w) top = fmaxf(top, sm_m[w * LAM_TOKENS + tok]);
-        float den = 0.f, o = 0.f;
+        const float sink2 = sink ? sink[head] * LA_LOG2E : -INFINITY;       // in units of log 2, like the maxima
+        top = fmaxf(top, sink2);
+        float den = __builtin_amdgcn_exp2f(sink2 - top), o = 0.f;           // (0 without a sink)
 #pragma unroll
         for (int w = 0; w < LAM_WAVES; ++w) {
             const float f = __builtin_amdgcn_exp2f(sm_m[w * LAM_TOKENS + tok] - top);        // (0 for a wave that saw no key of this token)
@@ -342,7 +369,8 @@ template <int DK, int DV>
 static void launch_local_mfma(const void* q, int q_ld, void* out, int out_ld, const void* k_plane, const void* v_plane, const void* block_table,
                               int table_ld, int table_width, const void* req_indptr, const void* ctx_lens, const void* tile_req,
                               const void* tile_tok0, int tiles, int heads, int kv_heads, int page_size, float scale, float cap, LocalMask mask,
-                              float gain, hipStream_t stream) {
+                              float gain, const void* sink, const void* pk_plane, const void* pv_plane, const void* pool_table, int pool_table_ld,
+                              int pool_table_width, int pool, hipStream_t stream) {
     dim3 grid(tiles, heads), block(LAM_WAVES * TL_WAVE);
     const size_t smem = sizeof(float) * LAM_WAVES * LAM_TOKENS * (2 + DV * 16);
     auto kernel = local_attention_mfma_kernel<DK, DV>;
@@ -353,7 +381,8 @@ static void launch_local_mfma(const void* q, int q_ld, void* out, int out_ld, co
     }
     kernel<<<grid, block, smem, stream>>>((const bf16_t*)q, q_ld, (bf16_t*)out, out_ld, (const bf16_t*)k_plane, (const bf16_t*)v_plane,
         (const int*)block_table, table_ld, table_width, (const int*)req_indptr, (const int*)ctx_lens, (const int*)tile_req, (const int*)tile_tok0,
-        heads, kv_heads, page_size, scale, cap, mask, gain);
+        heads, kv_heads, page_size, scale, cap, mask, gain, (const float*)sink, (const bf16_t*)pk_plane, (const bf16_t*)pv_plane, (const int*)pool_table,
+        pool_table_ld, pool_table_width, pool);
 }
 
 // Whether the matrix-core kernel is built for these sizes.
@@ -368,7 +397,11 @@ extern "C" int tl_local_attention_mfma_fits(int dim, int vdim, int page_size) {
 extern "C" int tl_local_attention_tiles(const void* q, int q_ld, void* out, int out_ld, const void* k_plane, const void* v_plane, int pages,
                                         const void* block_table, int table_ld, int table_width, const void* req_indptr, const void* ctx_lens,
                                         const void* tile_req, const void* tile_tok0, int tiles, int heads, int kv_heads, int dim, int vdim,
-                                        int page_size, float scale, float cap, int chunk, int window, float gain, hipStream_t stream) {
+                                        int page_size, float scale, float cap, int chunk, int window, float gain, const void* sink,
+                                        const void* pk_plane, const void* pv_plane, const void* pool_table, int pool_table_ld, int pool_table_width,
+                                        int pool, hipStream_t stream) {
+    TL_REQUIRE(pool >= 0 && (pool == 0 || (window > 0 && pk_plane && pv_plane && pool_table && pool_table_ld >= pool_table_width && pool_table_width > 0)),
+               "local_attention_tiles: pooled blocks need a window, their planes and their block table");
     TL_REQUIRE(tiles >= 0 && heads > 0 && heads <= 65535 && kv_heads > 0 && heads % kv_heads == 0 && page_size > 0, "local_attention_tiles: bad sizes");
     TL_REQUIRE(tl_local_attention_mfma_fits(dim, vdim, page_size), "local_attention_tiles: not built for heads of %d / %d numbers in pages of %d", dim, vdim, page_size);
     TL_REQUIRE(q_ld >= heads * dim && q_ld % 8 == 0 && ((uintptr_t)q & 15) == 0 && out_ld >= heads * vdim && table_ld >= table_width && chunk >= 0 && window >= 0,
@@ -377,7 +410,8 @@ extern "C" int tl_local_attention_tiles(const void* q, int q_ld, void* out, int 
     const LocalMask mask{chunk, window};
 #define TL_LAM(DK, DV)                                                                                                                      \
     launch_local_mfma<DK, DV>(q, q_ld, out, out_ld, k_plane, v_plane, block_table, table_ld, table_width, req_indptr, ctx_lens, tile_req,  \
-                              tile_tok0, tiles, heads, kv_heads, page_size, scale, cap, mask, gain, stream)
+                              tile_tok0, tiles, heads, kv_heads, page_size, scale, cap, mask, gain, sink, pk_plane, pv_plane, pool_table,        \
+                              pool_table_ld, pool_table_width, pool, stream)
 #define TL_LAM_V(DK)                                     \
     switch (vdim) {                                      \
         case 16: TL_LAM(DK, 1); break;                   \
@@ -405,7 +439,9 @@ extern "C" int tl_local_attention_tiles(const void* q, int q_ld, void* out, int 
 extern "C" int tl_local_attention(const void* q, int q_ld, void* out, int out_ld, const void* k_plane, const void* v_plane, int pages,
                                   const void* block_table, int table_ld, int table_width, const void* token_req, const void* positions,
                                   int tokens, int heads, int kv_heads, int dim, int vdim, int page_size, float scale, float cap, int chunk,
-                                  int window, float gain, int dtype, hipStream_t stream) {
+                                  int window, float gain, const void* sink, const void* pk_plane, const void* pv_plane, const void* pool_table,
+                                  int pool_table_ld, int pool, int dtype, hipStream_t stream) {
+    TL_REQUIRE(pool >= 0 && (pool == 0 || (window > 0 && pk_plane && pv_plane && pool_table)), "local_attention: pooled blocks need a window, their planes and their block table");
     TL_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0 && page_size > 0, "local_attention: bad sizes");
     TL_REQUIRE(dim <= LA_MAX_DIM && vdim <= LA_MAX_DIM, "local_attention: built for heads of up to %d numbers, got %d / %d", LA_MAX_DIM, dim, vdim);
     TL_REQUIRE(q_ld >= heads * dim && out_ld >= heads * vdim && table_ld >= table_width && chunk >= 0 && window >= 0, "local_attention: rows too short");
@@ -415,11 +451,141 @@ extern "C" int tl_local_attention(const void* q, int q_ld, void* out, int out_ld
     dim3 grid(tokens, heads), block(LA_WAVES * TL_WAVE);
     if (dtype == TL_DT_F32)
         local_attention_kernel<float><<<grid, block, 0, stream>>>((const float*)q, q_ld, (float*)out, out_ld, (const float*)k_plane, (const float*)v_plane,
-            (const int*)block_table, table_ld, (const int*)token_req, (const int*)positions, heads, kv_heads, dim, vdim, page_size, scale, cap, mask, gain);
+            (const int*)block_table, table_ld, (const int*)token_req, (const int*)positions, heads, kv_heads, dim, vdim, page_size, scale, cap, mask, gain,
+            (const float*)sink, (const float*)pk_plane, (const float*)pv_plane, (const int*)pool_table, pool_table_ld, pool);
     else if (dtype == TL_DT_BF16)
         local_attention_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)q, q_ld, (bf16_t*)out, out_ld, (const bf16_t*)k_plane, (const bf16_t*)v_plane,
-            (const int*)block_table, table_ld, (const int*)token_req, (const int*)positions, heads, kv_heads, dim, vdim, page_size, scale, cap, mask, gain);
+            (const int*)block_table, table_ld, (const int*)token_req, (const int*)positions, heads, kv_heads, dim, vdim, page_size, scale, cap, mask, gain,
+            (const float*)sink, (const bf16_t*)pk_plane, (const bf16_t*)pv_plane, (const int*)pool_table, pool_table_ld, pool);
     else TL_REQUIRE(false, "local_attention: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("local_attention");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ pooled blocks
+// Block b of a request (positions b * pool .. b * pool + pool - 1) gets its pooled key and value, the means of its cached keys and values,
+// in the step that brings its last token: the blocks ctx / pool .. (ctx + n) / pool - 1 of a request that held ctx tokens and gets n.  One
+// work-group per such block; sums in float in the order of the positions, one rounding.  Pooled rows lie in planes laid out like the
+// tokens' (values transposed) under a block table of their own, block b in row b; what would go to page 0 is dropped.
+template <typename T>
+__global__ void pool_blocks_kernel(const T* __restrict__ k_plane, const T* __restrict__ v_plane, const int* __restrict__ block_table, int table_ld,
+                                   int table_width, T* __restrict__ pk_plane, T* __restrict__ pv_plane, const int* __restrict__ pool_table,
+                                   int pool_table_ld, int pool_table_width, const int* __restrict__ req_indptr, const int* __restrict__ ctx_lens,
+                                   int kv_heads, int dim, int vdim, int pages, int pool_pages, int page_size, int pool) {
+    const int r = blockIdx.y;
+    const int ctx = ctx_lens[r], n = req_indptr[r + 1] - req_indptr[r];
+    const int b = ctx / pool + blockIdx.x;
+    if (n <= 0 || b >= (ctx + n) / pool) return;
+    const int pb = b / page_size;
+    if (pb >= pool_table_width) return;
+    const int ppage = pool_table[(size_t)r * pool_table_ld + pb];
+    if (ppage <= 0 || ppage >= pool_pages) return;
+    const int pslot = b % page_size;
+    const int* table = block_table + (size_t)r * table_ld;
+    const float inv = 1.f / (float)pool;
+    for (int i = threadIdx.x; i < kv_heads * (dim + vdim); i += blockDim.x) {
+        const bool is_key = i < kv_heads * dim;
+        const int e = is_key ? i : i - kv_heads * dim;
+        const int width = is_key ? dim : vdim;
+        const int g = e / width, d = e % width;
+        float sum = 0.f;
+        for (int j = 0; j < pool; ++j) {
+            const int key = b * pool + j, blk = key / page_size, slot = key % page_size;
+            const int page = blk < table_width ? table[blk] : 0;
+            if (page <= 0 || page >= pages) continue;          // (a block's tokens are all held when its last one arrives)
+            sum += is_key ? to_float(k_plane[(((size_t)page * kv_heads + g) * page_size + slot) * dim + d])
+                          : to_float(v_plane[(((size_t)page * kv_heads + g) * vdim + d) * page_size + slot]);
+        }
+        if (is_key) pk_plane[(((size_t)ppage * kv_heads + g) * page_size + pslot) * dim + d] = from_float<T>(sum * inv);
+        else pv_plane[(((size_t)ppage * kv_heads + g) * vdim + d) * page_size + pslot] = from_float<T>(sum * inv);
+    }
+}
+
+// `most_blocks`: an upper bound of the blocks one request completes in the step (its longest portion / pool + 1).
+extern "C" int tl_pool_blocks(const void* k_plane, const void* v_plane, int pages, const void* block_table, int table_ld, int table_width,
+                              void* pk_plane, void* pv_plane, int pool_pages, const void* pool_table, int pool_table_ld, int pool_table_width,
+                              const void* req_indptr, const void* ctx_lens, int requests, int most_blocks, int kv_heads, int dim, int vdim,
+                              int page_size, int pool, int dtype, hipStream_t stream) {
+    TL_REQUIRE(requests >= 0 && requests <= 65535 && most_blocks >= 0 && kv_heads > 0 && dim > 0 && vdim > 0 && page_size > 0 && pool > 0 && pages > 0 && pool_pages > 0,
+               "pool_blocks: bad sizes");
+    TL_REQUIRE(table_ld >= table_width && pool_table_ld >= pool_table_width && table_width > 0 && pool_table_width > 0, "pool_blocks: block tables too short");
+    if (requests == 0 || most_blocks == 0) return TL_OK;
+    dim3 grid(most_blocks, requests), block(256);
+    if (dtype == TL_DT_F32)
+        pool_blocks_kernel<float><<<grid, block, 0, stream>>>((const float*)k_plane, (const float*)v_plane, (const int*)block_table, table_ld, table_width,
+            (float*)pk_plane, (float*)pv_plane, (const int*)pool_table, pool_table_ld, pool_table_width, (const int*)req_indptr, (const int*)ctx_lens,
+            kv_heads, dim, vdim, pages, pool_pages, page_size, pool);
+    else if (dtype == TL_DT_BF16)
+        pool_blocks_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)k_plane, (const bf16_t*)v_plane, (const int*)block_table, table_ld, table_width,
+            (bf16_t*)pk_plane, (bf16_t*)pv_plane, (const int*)pool_table, pool_table_ld, pool_table_width, (const int*)req_indptr, (const int*)ctx_lens,
+            kv_heads, dim, vdim, pages, pool_pages, page_size, pool);
+    else TL_REQUIRE(false, "pool_blocks: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("pool_blocks");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ norm per head and rotation, in place
+// x [T, ld] holds per token heads_a + heads_b heads of `dim` numbers side by side (queries, then keys).  One wave per token and head, in float:
+//   norm (norm_a / norm_b != null): v <- v / sqrt(mean(v^2) + eps) * w[d], w = norm_a for the first heads_a heads, norm_b for the others;
+//   rotation (inv_freq != null) of the first `dims` numbers by angle_i = float(position) * inv_freq[i]: pair (2i, 2i + 1), or, `halves`,
+//   pair (i, i + dims / 2); (u, v) <- (u cos - v sin, v cos + u sin).  What lies beyond `dims` is not turned.  One rounding at the end.
+#define HNR_WAVES 4
+template <typename T>
+__global__ void __launch_bounds__(HNR_WAVES * TL_WAVE)
+head_norm_rotate_kernel(T* __restrict__ x, int ld, int tokens, int heads_a, int heads_b, int dim, const float* __restrict__ norm_a,
+                        const float* __restrict__ norm_b, float eps, const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                        int dims, int halves) {
+    __shared__ float sv[HNR_WAVES][LA_MAX_DIM];
+    const int wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
+    const int heads = heads_a + heads_b;
+    const long item = (long)blockIdx.x * HNR_WAVES + wave;
+    const bool live = item < (long)tokens * heads;
+    const int t = live ? (int)(item / heads) : 0, h = live ? (int)(item % heads) : 0;
+    T* row = x + (size_t)t * ld + (size_t)h * dim;
+    float* v = sv[wave];
+    const float* w = h < heads_a ? norm_a : norm_b;
+    float ss = 0.f;
+    if (live)
+        for (int d = lane; d < dim; d += TL_WAVE) { const float a = to_float(row[d]); v[d] = a; ss = fmaf(a, a, ss); }
+    ss = wave_sum(ss);
+    __syncthreads();
+    if (live && w) {
+        const float inv = 1.f / sqrtf(ss / (float)dim + eps);
+        for (int d = lane; d < dim; d += TL_WAVE) v[d] = v[d] * inv * w[d];
+    }
+    __syncthreads();
+    if (live && inv_freq) {
+        const float pos = (float)positions[t];
+        for (int i = lane; i < dims / 2; i += TL_WAVE) {
+            const int ia = halves ? i : 2 * i, ib = halves ? i + dims / 2 : 2 * i + 1;
+            float sn, c;
+            sincosf(pos * inv_freq[i], &sn, &c);
+            const float a = v[ia], b = v[ib];
+            v[ia] = __fmaf_rn(a, c, -__fmul_rn(b, sn));
+            v[ib] = __fmaf_rn(b, c, __fmul_rn(a, sn));
+        }
+    }
+    __syncthreads();
+    if (live)
+        for (int d = lane; d < dim; d += TL_WAVE) row[d] = from_float<T>(v[d]);
+}
+
+extern "C" int tl_head_norm_rotate(void* x, int ld, int tokens, int heads_a, int heads_b, int dim, const void* norm_a, const void* norm_b, float eps,
+                                   const void* positions, const void* inv_freq, int dims, int halves, int dtype, hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && heads_a >= 0 && heads_b >= 0 && heads_a + heads_b > 0 && dim > 0 && dim <= LA_MAX_DIM && ld >= (heads_a + heads_b) * dim,
+               "head_norm_rotate: bad sizes");
+    TL_REQUIRE(!inv_freq || (positions && dims > 0 && dims % 2 == 0 && dims <= dim), "head_norm_rotate: a rotation over %d of %d numbers", dims, dim);
+    TL_REQUIRE((norm_a == nullptr) == (norm_b == nullptr) || heads_a == 0 || heads_b == 0, "head_norm_rotate: a norm for both kinds of heads or for neither");
+    if (tokens == 0) return TL_OK;
+    const long items = (long)tokens * (heads_a + heads_b);
+    const int grid = (int)((items + HNR_WAVES - 1) / HNR_WAVES);
+    if (dtype == TL_DT_F32)
+        head_norm_rotate_kernel<float><<<grid, HNR_WAVES * TL_WAVE, 0, stream>>>((float*)x, ld, tokens, heads_a, heads_b, dim, (const float*)norm_a,
+            (const float*)norm_b, eps, (const int*)positions, (const float*)inv_freq, dims, halves);
+    else if (dtype == TL_DT_BF16)
+        head_norm_rotate_kernel<bf16_t><<<grid, HNR_WAVES * TL_WAVE, 0, stream>>>((bf16_t*)x, ld, tokens, heads_a, heads_b, dim, (const float*)norm_a,
+            (const float*)norm_b, eps, (const int*)positions, (const float*)inv_freq, dims, halves);
+    else TL_REQUIRE(false, "head_norm_rotate: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("head_norm_rotate");
     return TL_OK;
 }

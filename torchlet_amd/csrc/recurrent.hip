@@ -492,9 +492,12 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-template <int RPL, int TB>
+// DELTA false: the same recurrence without the correction, S <- g S + k v^T and o = S^T q, with one fixed decay per head (`head_decay`)
+// in place of the tokens' gates: the decayed linear attention.
+template <int RPL, int TB, bool DELTA>
 __global__ void __launch_bounds__(256)
-delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates, float* __restrict__ state, size_t slot_stride,
+delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates, const float* __restrict__ head_decay,
+                  float* __restrict__ state, size_t slot_stride,
                   const int* __restrict__ slots, const int* __restrict__ req_indptr, float* __restrict__ out,
                   int heads, int kv_heads, int dim, int vdim) {
     constexpr int tb = TB;
@@ -546,7 +549,8 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
                     if (e < ROWS) v = e < dim ? row[q_at + e] : 0.f;
                     else if (e < 2 * ROWS) v = e - ROWS < dim ? row[k_at + e - ROWS] : 0.f;
                     else if (e < 2 * ROWS + DELTA_COLS) v = col0 + e - 2 * ROWS < vdim ? row[v_at + e - 2 * ROWS] : 0.f;
-                    else v = gates[(size_t)(base + t) * 2 * heads + (e - 2 * ROWS - DELTA_COLS) * heads + head];
+                    else if (DELTA) v = gates[(size_t)(base + t) * 2 * heads + (e - 2 * ROWS - DELTA_COLS) * heads + head];
+                    else v = e == PER_TOKEN - 1 ? head_decay[head] : 1.f;
                 } else if (e == PER_TOKEN - 1) v = 1.f;        // beyond the request's last token: k = 0, beta = 0 and a decay of 1 leave the state as it is, to the bit
             }
             stage[j] = v;
@@ -590,14 +594,14 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
                 float a4[4] = {0.f, 0.f, 0.f, 0.f}, b4[4] = {0.f, 0.f, 0.f, 0.f}, c4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int r = 0; r < RPL; ++r) {
-                    a4[r & 3] = fmaf(S[r], kr[r], a4[r & 3]);
+                    if (DELTA) a4[r & 3] = fmaf(S[r], kr[r], a4[r & 3]);
                     b4[r & 3] = fmaf(S[r], qr[r], b4[r & 3]);
                     c4[r & 3] = fmaf(kr[r], qr[r], c4[r & 3]);
                 }
-                const float a = row16_sum((a4[0] + a4[1]) + (a4[2] + a4[3]));
+                const float a = DELTA ? row16_sum((a4[0] + a4[1]) + (a4[2] + a4[3])) : 0.f;
                 const float b = row16_sum((b4[0] + b4[1]) + (b4[2] + b4[3]));
                 const float kq = row16_sum((c4[0] + c4[1]) + (c4[2] + c4[3]));
-                const float u = beta * (vt - g * a);
+                const float u = DELTA ? beta * (vt - g * a) : vt;
 #pragma unroll
                 for (int r = 0; r < RPL; ++r) S[r] = fmaf(kr[r], u, g * S[r]);
                 obuf[t] = fmaf(kq, u, g * b);
@@ -621,21 +625,17 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
 }
 
 // state: per slot, from its start, heads x [vdim][dim] floats (a head's state column by column).
-extern "C" int tl_delta_scan(const void* qkv, const void* gates, void* state, long slot_stride, const void* slots, const void* req_indptr,
-                             void* out, int requests, int heads, int kv_heads, int dim, int vdim, int longest, hipStream_t stream) {
-    TL_REQUIRE(requests >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0, "delta_scan: bad sizes");
-    TL_REQUIRE(dim <= DELTA_L * 16, "delta_scan: built for up to %d query/key dimensions per head, got %d", DELTA_L * 16, dim);
-    TL_REQUIRE(slot_stride >= (long)heads * dim * vdim, "delta_scan: the state rows are too short");
-    TL_REQUIRE(requests <= 65535 && heads <= 65535, "delta_scan: too many requests or heads for one launch");
-    if (requests == 0) return TL_OK;
+template <bool DELTA>
+static int launch_delta_scan(const void* qkv, const void* gates, const void* head_decay, void* state, long slot_stride, const void* slots,
+                             const void* req_indptr, void* out, int requests, int heads, int kv_heads, int dim, int vdim, int longest, hipStream_t stream) {
     const int rpl = dim <= 64 ? 4 : dim <= 128 ? 8 : dim <= 192 ? 12 : 16;
     // tokens of a batch: 1 for a step of single tokens, 4 for short portions, else 16 (a batch is always worked through whole)
     const int tb = longest <= 1 ? 1 : (longest <= 4 ? 4 : DELTA_TB);
     const size_t smem = sizeof(float) * (size_t)tb * (2 * DELTA_L * rpl + DELTA_COLS + 2);
     dim3 grid((vdim + DELTA_COLS - 1) / DELTA_COLS, heads, requests), block(256);
 #define TL_DELTA_B(R, B)                                                                                                                   \
-    delta_scan_kernel<R, B><<<grid, block, smem, stream>>>((const float*)qkv, (const float*)gates, (float*)state, (size_t)slot_stride,    \
-                                                           (const int*)slots, (const int*)req_indptr, (float*)out, heads, kv_heads, dim, vdim)
+    delta_scan_kernel<R, B, DELTA><<<grid, block, smem, stream>>>((const float*)qkv, (const float*)gates, (const float*)head_decay, (float*)state, \
+                                                           (size_t)slot_stride, (const int*)slots, (const int*)req_indptr, (float*)out, heads, kv_heads, dim, vdim)
 #define TL_DELTA(R)                        \
     if (tb == 1) TL_DELTA_B(R, 1);         \
     else if (tb == 4) TL_DELTA_B(R, 4);    \
@@ -646,6 +646,53 @@ extern "C" int tl_delta_scan(const void* qkv, const void* gates, void* state, lo
     else { TL_DELTA(16); }
 #undef TL_DELTA
 #undef TL_DELTA_B
+    return TL_OK;
+}
+
+extern "C" int tl_delta_scan(const void* qkv, const void* gates, void* state, long slot_stride, const void* slots, const void* req_indptr,
+                             void* out, int requests, int heads, int kv_heads, int dim, int vdim, int longest, hipStream_t stream) {
+    TL_REQUIRE(requests >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0, "delta_scan: bad sizes");
+    TL_REQUIRE(dim <= DELTA_L * 16, "delta_scan: built for up to %d query/key dimensions per head, got %d", DELTA_L * 16, dim);
+    TL_REQUIRE(slot_stride >= (long)heads * dim * vdim, "delta_scan: the state rows are too short");
+    TL_REQUIRE(requests <= 65535 && heads <= 65535, "delta_scan: too many requests or heads for one launch");
+    if (requests == 0) return TL_OK;
+    launch_delta_scan<true>(qkv, gates, nullptr, state, slot_stride, slots, req_indptr, out, requests, heads, kv_heads, dim, vdim, longest, stream);
     TL_CHECK_LAUNCH("delta_scan");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ decayed linear attention
+// Per head S <- decay[head] S + k v^T, o = S^T q over the step's tokens, request by request from the state its slot holds: qkv float
+// [T, 2 * heads * dim + heads * vdim] (queries, keys, values, head by head), state as the delta rule's, out float [T, heads * vdim].
+extern "C" int tl_decay_scan(const void* qkv, const void* decay, void* state, long slot_stride, const void* slots, const void* req_indptr,
+                             void* out, int requests, int heads, int dim, int vdim, int longest, hipStream_t stream) {
+    TL_REQUIRE(requests >= 0 && heads > 0 && dim > 0 && vdim > 0 && decay, "decay_scan: bad sizes");
+    TL_REQUIRE(dim <= DELTA_L * 16, "decay_scan: built for up to %d query/key dimensions per head, got %d", DELTA_L * 16, dim);
+    TL_REQUIRE(slot_stride >= (long)heads * dim * vdim, "decay_scan: the state rows are too short");
+    TL_REQUIRE(requests <= 65535 && heads <= 65535, "decay_scan: too many requests or heads for one launch");
+    if (requests == 0) return TL_OK;
+    launch_delta_scan<false>(qkv, nullptr, decay, state, slot_stride, slots, req_indptr, out, requests, heads, heads, dim, vdim, longest, stream);
+    TL_CHECK_LAUNCH("decay_scan");
+    return TL_OK;
+}
+
+// out[t, c] = silu(float(x[t, c])) for the first `cols` columns of every row (the rows of x may be longer).
+template <typename T>
+__global__ void silu_float_kernel(const T* __restrict__ x, int ld, float* __restrict__ out, int cols, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const float v = to_float(x[(i / cols) * ld + i % cols]);
+    out[i] = v / (1.f + expf(-v));
+}
+
+extern "C" int tl_silu_float(const void* x, int ld, void* out, int rows, int cols, int dtype, hipStream_t stream) {
+    TL_REQUIRE(rows >= 0 && cols > 0 && ld >= cols, "silu_float: bad sizes");
+    if (rows == 0) return TL_OK;
+    const size_t total = (size_t)rows * cols;
+    const int grid = (int)((total + 255) / 256);
+    if (dtype == TL_DT_F32) silu_float_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, ld, (float*)out, cols, total);
+    else if (dtype == TL_DT_BF16) silu_float_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, ld, (float*)out, cols, total);
+    else TL_REQUIRE(false, "silu_float: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("silu_float");
     return TL_OK;
 }

@@ -42,7 +42,7 @@ class ModelRunner:
         self.model = model
         self.cache = cache
         self.device = model.device
-        self.caches = [cache.layer_cache(i) for i in range(len(model.spec.order))]
+        self.caches = [cache.layer_cache(i) for i in range(len(model.cache_plan()))]      # the runs' caches, then the model's own state if it keeps one
         self.tile_sizes = model.tile_token_sizes()
         self.max_positions = model.spec.max_positions if max_model_len is None else min(max_model_len, model.spec.max_positions)
         self.vocab_size = model.spec.vocab_size

@@ -143,6 +143,77 @@ def embedding(token_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, s
                                  c_int(copies), _stream()))
 
 
+def bigram_embedding(token_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float, bigram: torch.Tensor, buckets: int,
+                     mul_prev: int, mul_cur: int, token_req: torch.Tensor, req_indptr: torch.Tensor, positions: torch.Tensor,
+                     slots: torch.Tensor, last_token: torch.Tensor) -> None:
+    """``out[t] = float(table[token_ids[t]]) * scale + float(bigram[row(t)])`` with ``row(t) = (previous token * mul_prev + token * mul_cur) mod
+    buckets``, or ``buckets`` for a token at position 0.  The token before a request's first token of the step is ``last_token[slot]`` (int32
+    ``[slots, 1]``), where the step then leaves the request's last token.  ``out`` is the 32-bit residual ``[T, H]`` or ``[copies, T, H]``."""
+    T = token_ids.numel()
+    V, H = table.shape
+    R = req_indptr.numel() - 1
+    _i32(token_ids, "embedding ids", T)
+    _i32(token_req, "token_req", T)
+    _i32(positions, "positions", T)
+    _i32(req_indptr, "req_indptr", R + 1)
+    _i32(slots, "slots", R)
+    copies = out.shape[0] if out.dim() == 3 else 1
+    if out.shape[-2:] != (T, H) or out.dim() not in (2, 3) or out.dtype != torch.float32 or not out.is_contiguous() or not table.is_contiguous():
+        raise KernelError(f"bigram_embedding: out must be contiguous float32 [{T}, {H}] or [copies, {T}, {H}], got {out.dtype} {tuple(out.shape)}")
+    if bigram.shape != (buckets + 1, H) or bigram.dtype != table.dtype or not bigram.is_contiguous() or buckets <= 0:
+        raise KernelError(f"bigram_embedding: the bigram table must be [{buckets + 1}, {H}] of {table.dtype}")
+    if last_token.dtype != torch.int32 or not last_token.is_contiguous() or last_token.dim() != 2 or last_token.shape[1] != 1:
+        raise KernelError("bigram_embedding: the requests' last tokens are int32 [slots, 1]")
+    lib = _lib("elementwise")
+    _check(lib, lib.tl_bigram_embedding(_ptr(token_ids), _ptr(table), _ptr(out), c_int(T), c_int(H), c_int(V), c_float(scale), _ptr(token_req),
+                                        _ptr(req_indptr), c_int(R), _ptr(positions), _ptr(slots), _ptr(last_token), _ptr(bigram), c_int(buckets),
+                                        ctypes.c_long(mul_prev), ctypes.c_long(mul_cur), c_int(copies), c_int(_dt(table, "embedding table")), _stream()))
+
+
+def sandwich_norm(residual: torch.Tensor, pending: torch.Tensor | None, post_weight: torch.Tensor | None, post_eps: float,
+                  extra: torch.Tensor | None, weight: torch.Tensor, eps: float, out: torch.Tensor, rows: torch.Tensor | None = None,
+                  gain: float = 1.0) -> None:
+    """``r = residual (+ extra) + (pending / sqrt(mean(pending^2) + post_eps) * post_weight, or pending as it is without a post_weight)``, written
+    back to the float32 residual ``[T, H]`` unless ``rows`` selects rows; ``out = r / sqrt(mean(r^2) + eps) * weight * gain`` in its own dtype.
+    ``pending``: ``[T, H]`` of ``out``'s dtype or float32 slabs ``[P, T, H]`` that are added up; ``extra``: float32 ``[T, H]``; ``weight`` and
+    ``post_weight``: float32, one number or ``H`` of them."""
+    T, H = residual.shape
+    if residual.dtype != torch.float32 or not residual.is_contiguous():
+        raise KernelError("sandwich_norm: the residual must be contiguous float32")
+    n = T if rows is None else rows.numel()
+    _i32(rows, "rows", n)
+    if out.shape != (n, H) or not out.is_contiguous():
+        raise KernelError(f"sandwich_norm: out must be contiguous [{n}, {H}], got {tuple(out.shape)}")
+    parts = 0
+    if pending is not None:
+        if pending.dim() == 3:
+            parts = pending.shape[0]
+            if pending.dtype != torch.float32 or pending.shape[1:] != residual.shape or not pending.is_contiguous():
+                raise KernelError(f"sandwich_norm: partial sums {pending.dtype} {tuple(pending.shape)} are not float32 [P, {T}, {H}]")
+        elif pending.shape != residual.shape or pending.dtype != out.dtype or not pending.is_contiguous():
+            raise KernelError(f"sandwich_norm: pending {pending.dtype} {tuple(pending.shape)} does not match the residual and the output's dtype")
+    if extra is not None and (extra.dtype != torch.float32 or extra.shape != residual.shape or not extra.is_contiguous()):
+        raise KernelError("sandwich_norm: the second addend must be contiguous float32 like the residual")
+    for w, what in ((weight, "weight"), (post_weight, "post_weight")):
+        if w is not None and (w.dtype != torch.float32 or not w.is_contiguous() or w.numel() not in (1, H)):
+            raise KernelError(f"sandwich_norm: {what} must be float32, one number or {H}")
+    lib = _lib("elementwise")
+    _check(lib, lib.tl_sandwich_norm(_ptr(residual), _ptr(pending), c_int(parts), c_int(T), _ptr(post_weight if pending is not None else None),
+                                     c_int(post_weight.numel() if post_weight is not None else 0), c_float(post_eps), _ptr(extra), _ptr(weight),
+                                     c_int(weight.numel()), c_float(eps), c_float(gain), _ptr(out), _ptr(rows), c_int(n), c_int(H),
+                                     c_int(_dt(out, "sandwich_norm")), _stream()))
+
+
+def normed_sum(x: torch.Tensor, weights: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """``out[t] = sum_b x[b, t] / sqrt(mean(x[b, t]^2) + eps) * weights[b]``: ``x [B, T, H]`` and ``out [T, H]`` of one dtype, ``weights`` float32 ``[B, H]``."""
+    B, T, H = x.shape
+    if not x.is_contiguous() or out.shape != (T, H) or out.dtype != x.dtype or not out.is_contiguous() \
+            or weights.dtype != torch.float32 or weights.shape != (B, H) or not weights.is_contiguous():
+        raise KernelError("normed_sum: shapes or dtypes do not fit")
+    lib = _lib("elementwise")
+    _check(lib, lib.tl_normed_sum(_ptr(x), c_int(B), c_int(T), c_int(H), _ptr(weights), c_float(eps), _ptr(out), c_int(_dt(x, "normed_sum")), _stream()))
+
+
 NORM_KINDS = {"rmsnorm": 0, "layernorm": 1}
 MAX_STREAMS = 8
 
@@ -922,6 +993,39 @@ def delta_scan(qkv: torch.Tensor, gates: torch.Tensor, state: torch.Tensor, slot
                                   c_int(max(1, T - R + 1) if max_new_tokens is None else max_new_tokens), _stream()))
 
 
+def decay_scan(qkv: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, slots: torch.Tensor, req_indptr: torch.Tensor, out: torch.Tensor,
+               heads: int, dim: int, vdim: int, max_new_tokens: int | None = None) -> None:
+    """Linear attention with one fixed decay per head over the step's tokens, request by request from the state its slot holds: ``qkv``
+    float32 ``[T, 2 * heads * dim + heads * vdim]`` (queries, keys, values, head by head), ``decay`` float32 ``[heads]``; head ``h`` of
+    ``state[slot]`` (float32, laid out as :func:`delta_scan`'s) moves by ``S <- decay[h] S + k v^T`` and ``out`` float32 ``[T, heads * vdim]``
+    receives ``S^T q``."""
+    T = qkv.shape[0]
+    R = req_indptr.numel() - 1
+    C = 2 * heads * dim + heads * vdim
+    if qkv.dtype != torch.float32 or qkv.shape != (T, C) or not qkv.is_contiguous():
+        raise KernelError(f"decay_scan: qkv must be contiguous float32 [{T}, {C}]")
+    if decay.dtype != torch.float32 or decay.shape != (heads,) or not decay.is_contiguous():
+        raise KernelError(f"decay_scan: decay must be contiguous float32 [{heads}]")
+    if out.dtype != torch.float32 or out.shape != (T, heads * vdim) or not out.is_contiguous():
+        raise KernelError(f"decay_scan: out must be contiguous float32 [{T}, {heads * vdim}]")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < heads * dim * vdim or dim > DELTA_MAX_DIM:
+        raise KernelError(f"decay_scan: state {tuple(state.shape)} does not hold {heads} states of {dim} x {vdim} (up to {DELTA_MAX_DIM} rows)")
+    _i32(slots, "slots", R)
+    _i32(req_indptr, "req_indptr", R + 1)
+    lib = _lib("recurrent")
+    _check(lib, lib.tl_decay_scan(_ptr(qkv), _ptr(decay), _ptr(state), ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(req_indptr), _ptr(out),
+                                  c_int(R), c_int(heads), c_int(dim), c_int(vdim),
+                                  c_int(max(1, T - R + 1) if max_new_tokens is None else max_new_tokens), _stream()))
+
+
+def silu_float(x: torch.Tensor, out: torch.Tensor) -> None:
+    """``out = silu(float32(x))``: ``x [T, C]`` a row-strided view of either dtype, ``out`` contiguous float32 ``[T, C]``."""
+    if x.dim() != 2 or x.stride(1) != 1 or out.dtype != torch.float32 or out.shape != x.shape or not out.is_contiguous():
+        raise KernelError("silu_float: x must be [T, C] with unit stride along C and out contiguous float32 of the same shape")
+    lib = _lib("recurrent")
+    _check(lib, lib.tl_silu_float(_ptr(x), c_int(x.stride(0)), _ptr(out), c_int(x.shape[0]), c_int(x.shape[1]), c_int(_dt(x, "silu_float")), _stream()))
+
+
 # ------------------------------------------------------------- attention with two head sizes, a cap and a local mask
 
 LOCAL_ATTENTION_MAX_DIM = 256
@@ -966,16 +1070,30 @@ def local_attention_mfma_fits(dtype: torch.dtype, dim: int, vdim: int, page_size
 
 def local_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v_plane: torch.Tensor, block_table: torch.Tensor,
                     token_req: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, page_size: int,
-                    scale: float, softcap: float = 0.0, chunk: int = 0, window: int = 0, gain: float = 1.0, tiles=None) -> None:
+                    scale: float, softcap: float = 0.0, chunk: int = 0, window: int = 0, gain: float = 1.0, tiles=None,
+                    sink: torch.Tensor | None = None, pooled=None) -> None:
     """Attention of the step's queries ``q [T, heads * dim]`` over their requests' cached keys and values (which hold the step's own tokens
     already): query head ``i`` reads key/value head ``i // (heads / kv_heads)``; ``score = q . k * scale``, then (``softcap > 0``) ``softcap *
     tanh(score / softcap)``; a query at position ``p`` reads the keys ``j <= p`` with ``j // chunk == p // chunk`` (``chunk > 0``) and ``j > p -
     window`` (``window > 0``); softmax and weighted sum in 32-bit; ``out [T, heads * vdim]`` receives the result times ``gain``.  ``q`` and ``out``
     may be row-strided views.  Without ``tiles`` one work-group per token and head walks the keys (every dtype and size).  ``tiles =
     (req_indptr, ctx_lens, tile_req, tile_tok0, number of tiles)`` (tiles of up to 16 consecutive tokens of one request, as a step
-    context makes them) runs the matrix-core kernel, where :func:`local_attention_mfma_fits` says it is built."""
+    context makes them) runs the matrix-core kernel, where :func:`local_attention_mfma_fits` says it is built.  ``sink`` (float32 ``[heads]``):
+    ``exp(sink[head])`` joins the softmax's denominator.  ``pooled = (pk_plane, pv_plane, pool_table, pool)`` (with a window): a query at
+    ``p`` also reads the rows ``0 .. (p - window + 1) // pool - 1`` of these planes (laid out like the tokens', with a block table of their own)."""
     T = q.shape[0]
     _check_local_planes("local_attention", k_plane, v_plane, q.dtype, kv_heads, dim, vdim, page_size)
+    if sink is not None and (sink.dtype != torch.float32 or sink.shape != (heads,) or not sink.is_contiguous()):
+        raise KernelError(f"local_attention: the sink must be contiguous float32 [{heads}]")
+    pk_plane = pv_plane = pool_table = None
+    pool = 0
+    if pooled is not None:
+        pk_plane, pv_plane, pool_table, pool = pooled
+        _check_local_planes("local_attention (pooled)", pk_plane, pv_plane, q.dtype, kv_heads, dim, vdim, page_size)
+        if pool <= 0 or window <= 0 or pool_table.dtype != torch.int32 or pool_table.dim() != 2 or pool_table.stride(1) != 1 \
+                or pool_table.shape[0] != block_table.shape[0]:
+            raise KernelError("local_attention: pooled blocks need a window, a block size and an int32 block table [requests, blocks]")
+    pool_args = (_ptr(sink), _ptr(pk_plane), _ptr(pv_plane), _ptr(pool_table), c_int(pool_table.stride(0) if pool else 0))
     if q.shape != (T, heads * dim) or out.shape != (T, heads * vdim) or q.stride(1) != 1 or out.stride(1) != 1 or out.dtype != q.dtype \
             or heads % kv_heads or max(dim, vdim) > LOCAL_ATTENTION_MAX_DIM:
         raise KernelError("local_attention: queries or output do not fit")
@@ -997,14 +1115,68 @@ def local_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
                                                  c_int(k_plane.shape[0]), _ptr(block_table), c_int(block_table.stride(0)), c_int(block_table.shape[1]),
                                                  _ptr(req_indptr), _ptr(ctx_lens), _ptr(tile_req), _ptr(tile_tok0), c_int(n_tiles), c_int(heads),
                                                  c_int(kv_heads), c_int(dim), c_int(vdim), c_int(page_size), c_float(scale), c_float(softcap),
-                                                 c_int(chunk), c_int(window), c_float(gain), _stream()))
+                                                 c_int(chunk), c_int(window), c_float(gain), *pool_args, c_int(pool_table.shape[1] if pool else 0),
+                                                 c_int(pool), _stream()))
         return
     _i32(token_req, "token_req", T)
     _i32(positions, "positions", T)
     _check(lib, lib.tl_local_attention(_ptr(q), c_int(q.stride(0)), _ptr(out), c_int(out.stride(0)), _ptr(k_plane), _ptr(v_plane), c_int(k_plane.shape[0]),
                                        _ptr(block_table), c_int(block_table.stride(0)), c_int(block_table.shape[1]), _ptr(token_req), _ptr(positions),
                                        c_int(T), c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim), c_int(page_size), c_float(scale),
-                                       c_float(softcap), c_int(chunk), c_int(window), c_float(gain), c_int(_dt(q, "local_attention")), _stream()))
+                                       c_float(softcap), c_int(chunk), c_int(window), c_float(gain), *pool_args, c_int(pool),
+                                       c_int(_dt(q, "local_attention")), _stream()))
+
+
+def pool_blocks(k_plane: torch.Tensor, v_plane: torch.Tensor, block_table: torch.Tensor, pk_plane: torch.Tensor, pv_plane: torch.Tensor,
+                pool_table: torch.Tensor, req_indptr: torch.Tensor, ctx_lens: torch.Tensor, most_blocks: int, page_size: int, pool: int) -> None:
+    """The pooled rows of the blocks of ``pool`` positions whose last token this step brought: for request ``r``, which held ``ctx_lens[r]``
+    tokens and got ``req_indptr[r + 1] - req_indptr[r]``, the blocks ``ctx // pool .. (ctx + n) // pool - 1``; row ``b`` of ``pk_plane`` / ``pv_plane``
+    (through ``pool_table``) receives the means of the cached keys and values of the positions ``b * pool .. b * pool + pool - 1`` (summed in
+    32-bit, rounded once).  ``most_blocks``: an upper bound of the blocks one request completes in the step."""
+    kv_heads, dim, vdim = k_plane.shape[1], k_plane.shape[3], v_plane.shape[2]
+    _check_local_planes("pool_blocks", k_plane, v_plane, k_plane.dtype, kv_heads, dim, vdim, page_size)
+    _check_local_planes("pool_blocks (pooled)", pk_plane, pv_plane, k_plane.dtype, kv_heads, dim, vdim, page_size)
+    R = req_indptr.numel() - 1
+    for t, what in ((block_table, "block table"), (pool_table, "pooled block table")):
+        if t.dtype != torch.int32 or t.dim() != 2 or t.stride(1) != 1 or t.shape[0] < R:
+            raise KernelError(f"pool_blocks: the {what} must be int32 [requests, blocks]")
+    _i32(req_indptr, "req_indptr", R + 1)
+    _i32(ctx_lens, "ctx_lens", R)
+    if pool <= 0 or most_blocks < 0:
+        raise KernelError("pool_blocks: a block holds at least one position")
+    lib = _lib("local_attention")
+    _check(lib, lib.tl_pool_blocks(_ptr(k_plane), _ptr(v_plane), c_int(k_plane.shape[0]), _ptr(block_table), c_int(block_table.stride(0)),
+                                   c_int(block_table.shape[1]), _ptr(pk_plane), _ptr(pv_plane), c_int(pk_plane.shape[0]), _ptr(pool_table),
+                                   c_int(pool_table.stride(0)), c_int(pool_table.shape[1]), _ptr(req_indptr), _ptr(ctx_lens), c_int(R),
+                                   c_int(most_blocks), c_int(kv_heads), c_int(dim), c_int(vdim), c_int(page_size), c_int(pool),
+                                   c_int(_dt(k_plane, "pool_blocks")), _stream()))
+
+
+def head_norm_rotate(x: torch.Tensor, heads_a: int, heads_b: int, dim: int, norm_a: torch.Tensor | None, norm_b: torch.Tensor | None, eps: float,
+                     positions: torch.Tensor | None, inv_freq: torch.Tensor | None, dims: int, halves: bool) -> None:
+    """In place on ``x [T, (heads_a + heads_b) * dim]`` (a row-strided view: queries, then keys), per token and head, in 32-bit with one rounding:
+    a root-mean-square norm over the head's ``dim`` numbers with the weight ``norm_a`` (the first ``heads_a`` heads) or ``norm_b`` (float32
+    ``[dim]``; ``None``: no norm), then the rotation of the first ``dims`` numbers by ``float32(position) * inv_freq[i]`` (float32 ``[dims / 2]``;
+    ``None``: no rotation), pairing ``2i`` with ``2i + 1`` or, ``halves``, ``i`` with ``i + dims / 2``."""
+    T = x.shape[0]
+    heads = heads_a + heads_b
+    if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] != heads * dim or dim > LOCAL_ATTENTION_MAX_DIM:
+        raise KernelError(f"head_norm_rotate: x {tuple(x.shape)} is not [T, {heads} heads of {dim}] (up to {LOCAL_ATTENTION_MAX_DIM} numbers a head)")
+    for w in (norm_a, norm_b):
+        if w is not None and (w.dtype != torch.float32 or w.shape != (dim,) or not w.is_contiguous()):
+            raise KernelError(f"head_norm_rotate: a norm's weight must be contiguous float32 [{dim}]")
+    if (norm_a is None) != (norm_b is None) and heads_a and heads_b:
+        raise KernelError("head_norm_rotate: a norm for both kinds of heads or for neither")
+    if inv_freq is not None:
+        if dims <= 0 or dims % 2 or dims > dim or inv_freq.dtype != torch.float32 or inv_freq.shape != (dims // 2,) or not inv_freq.is_contiguous():
+            raise KernelError(f"head_norm_rotate: a rotation over {dims} of {dim} numbers needs float32 frequencies [{dims // 2}]")
+        _i32(positions, "positions", T)
+        if positions is None:
+            raise KernelError("head_norm_rotate: a rotation needs the tokens' positions")
+    lib = _lib("local_attention")
+    _check(lib, lib.tl_head_norm_rotate(_ptr(x), c_int(x.stride(0)), c_int(T), c_int(heads_a), c_int(heads_b), c_int(dim), _ptr(norm_a), _ptr(norm_b),
+                                        c_float(eps), _ptr(positions if inv_freq is not None else None), _ptr(inv_freq), c_int(dims if inv_freq is not None else 0),
+                                        c_int(1 if halves else 0), c_int(_dt(x, "head_norm_rotate")), _stream()))
 
 
 # ------------------------------------------------------------- attention over a cached latent
@@ -1121,7 +1293,7 @@ def latent_attention(q: torch.Tensor, out: torch.Tensor, plane: torch.Tensor, bl
 # ------------------------------------------------------------- products over groups, routing
 
 # ``*_pairs``: the product's columns come in pairs (gate, up) and the output, half as wide, is ``act(gate) * up``
-ACTIVATIONS = {"none": 0, "relu2": 1, "silu": 2, "gelu_tanh": 3, "relu2_pairs": 17, "silu_pairs": 18, "gelu_tanh_pairs": 19}
+ACTIVATIONS = {"none": 0, "relu2": 1, "silu": 2, "gelu_tanh": 3, "gelu": 4, "relu2_pairs": 17, "silu_pairs": 18, "gelu_tanh_pairs": 19, "gelu_pairs": 20}
 
 
 def heads_linear(x: torch.Tensor, x_head: int, weight: torch.Tensor, out: torch.Tensor, out_head: int, general: bool = False) -> None:

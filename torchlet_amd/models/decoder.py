@@ -1,6 +1,7 @@
 """A decoder built from a :class:`~torchlet_amd.config.base.ModelSpec`.
 
-embedding (times ``embed_scale``, plus the position's row of a learned table if the specification names one) -> the runs of the layer order -> final norm on the wanted rows
+embedding (times ``embed_scale``, plus the position's row of a learned table if the specification names one, plus a hashed bigram row if
+it names one) -> the runs of the layer order (before a run that says so the embedding's output enters the stream again) -> final norm on the wanted rows
 (times ``logit_scale``) -> LM head (plus its bias, if the specification says it has one)
 (/root/reference/src/torchlet/v10_triton_paged_gqa/model/qwen2_5.py:55-87, where the factors are 1 and
 there is no bias).  The class
@@ -13,7 +14,7 @@ import torch
 
 from ..config.base import ModelSpec
 from ..kernels import ops
-from ..parts import BLOCKS, NORMS, Stream, WeightSpec
+from ..parts import BLOCKS, NORMS, StateNeed, Stream, WeightSpec
 from ..parts.base import KEEP_COMPUTE, KEEP_STORED, join_name, place, under
 
 
@@ -30,6 +31,12 @@ class DecoderModel:
         self.head: torch.Tensor | None = None
         self.head_bias: torch.Tensor | None = None
         self.position_table: torch.Tensor | None = None
+        self.bigram_table: torch.Tensor | None = None
+        self.keeps_embedding = any(e.add_embedding for e in spec.order)
+        if (spec.bigram is not None or self.keeps_embedding) and spec.streams:
+            raise ValueError("a bigram embedding or an embedding that enters the stream again runs over one plain residual")
+        if spec.bigram is not None and spec.position_table_name:
+            raise ValueError("a bigram embedding beside a learned position table is not built")
 
     # ------------------------------------------------------------------ weights
     def weight_specs(self) -> dict[str, WeightSpec]:
@@ -37,6 +44,8 @@ class DecoderModel:
         specs = {join_name(s.embed_name, s.weight_suffix): WeightSpec((s.vocab_size, s.hidden))}
         if s.position_table_name:
             specs[join_name(s.position_table_name, s.weight_suffix)] = WeightSpec((s.max_positions, s.hidden), keep=KEEP_STORED)
+        if s.bigram is not None:
+            specs[join_name(s.bigram.name, s.weight_suffix)] = WeightSpec((s.bigram.buckets + 1, s.hidden))
         for i, block in enumerate(self.blocks):
             for k, v in block.weight_specs().items():
                 specs[join_name(s.layer_name(i), k)] = v
@@ -53,6 +62,8 @@ class DecoderModel:
         self.embed = place(tensors[join_name(s.embed_name, s.weight_suffix)], KEEP_COMPUTE, self.dtype, self.device)
         if s.position_table_name:
             self.position_table = place(tensors[join_name(s.position_table_name, s.weight_suffix)], KEEP_STORED, self.dtype, self.device)
+        if s.bigram is not None:
+            self.bigram_table = place(tensors[join_name(s.bigram.name, s.weight_suffix)], KEEP_COMPUTE, self.dtype, self.device)
         for i, block in enumerate(self.blocks):      # (`tensors` may read from disk on access: each name is touched once)
             block.load_weights(under(tensors, s.layer_name(i)))
         self.final_norm.load_weights(under(tensors, s.final_norm_name))
@@ -65,11 +76,14 @@ class DecoderModel:
 
     # ------------------------------------------------------------------ cache needs
     def cache_plan(self):
-        """Per run of the order: ``(paged need, state need, cache_of)``."""
+        """Per run of the order: ``(paged need, state need, cache_of)``; a model whose embedding reads the token before keeps it as one
+        more entry after the runs: an int32 per request."""
         plan = []
         for e in self.spec.order:
             mixer = self.blocks[e.layer].mixer
             plan.append((mixer.paged_need(), mixer.state_need(), e.cache_of))
+        if self.spec.bigram is not None:
+            plan.append((None, StateNeed(shape=(1,), dtype=torch.int32), None))
         return plan
 
     def tile_token_sizes(self) -> set[int]:
@@ -101,11 +115,23 @@ class DecoderModel:
         T = ctx.num_tokens
         # the 32-bit residual, or the copies of it that blocks joined by hyper-connections keep: all start as the embedding's output
         shape = (self.spec.streams, T, self.spec.hidden) if self.spec.streams else (T, self.spec.hidden)
+        if self.keeps_embedding:            # a second copy of the embedding's output, for the runs before which it enters the stream again
+            shape = (2, T, self.spec.hidden)
         residual = torch.empty(shape, dtype=torch.float32, device=self.device)
-        ops.embedding(ctx.token_ids, self.embed, residual, self.spec.embed_scale,
-                      *((ctx.positions, self.position_table) if self.position_table is not None else ()))
+        big = self.spec.bigram
+        if big is not None:
+            ops.bigram_embedding(ctx.token_ids, self.embed, residual, self.spec.embed_scale, self.bigram_table, big.buckets, big.mul_prev,
+                                 big.mul_cur, ctx.token_req, ctx.req_indptr, ctx.positions, ctx.slots, caches[len(self.spec.order)].state)
+        else:
+            ops.embedding(ctx.token_ids, self.embed, residual, self.spec.embed_scale,
+                          *((ctx.positions, self.position_table) if self.position_table is not None else ()))
+        embedded = None
+        if self.keeps_embedding:
+            residual, embedded = residual[0], residual[1]
         stream = Stream(residual)
         for i, e in enumerate(self.spec.order):
+            if e.add_embedding:             # the next norm adds it beside the pending branch output
+                stream.extra = embedded
             stream = self.blocks[e.layer].forward(stream, ctx, caches[i])
         if ctx.want_rows is None or ctx.num_wanted == 0:
             return None

@@ -164,13 +164,16 @@ class PagedNeed:
     plane, for planes that differ (a compressed latent beside a small rotated part).  ``dtype``: the
     planes' element type; ``None`` is the model's.  Layers with equal needs share a group of pages.  ``chunk``: a query reads only
     keys of its own chunk of ``chunk`` positions (counted from position 0), so pages that lie wholly before the chunk of the next
-    position are kept no longer."""
+    position are kept no longer.  ``stride``: the planes hold one row for every ``stride`` positions (row ``p // stride``: a summary of a
+    block of tokens), so a page of them spans ``stride`` times as many positions.  A mixer that keeps rows at two rates (tokens inside
+    a window, summaries of what lies before it) declares two needs, each a group of its own."""
     num_heads: int
     head_dim: int
     window: int | None = None
     planes: int | tuple[tuple[int, int], ...] = 2
     dtype: torch.dtype | None = None
     chunk: int | None = None
+    stride: int = 1
 
     @property
     def bounded(self) -> bool:
@@ -210,15 +213,22 @@ class Stream:
 
     Blocks that keep several copies of the residual (hyper-connections) hold them as ``residual [S, T, hidden]``; ``fold`` then says
     how the pending output enters them: ``(mix [S, S], out [S])``, 32-bit tensors on the GPU, for ``x_t <- sum_s mix[s, t] x_s +
-    out[t] * pending`` (``None``: ``pending`` is added to every stream as it is)."""
+    out[t] * pending`` (``None``: ``pending`` is added to every stream as it is).
 
-    __slots__ = ("residual", "pending", "normed", "fold")
+    Blocks that norm a branch's output before it is added leave that norm on the stream as well: ``post = (weight, eps)`` means that
+    ``pending`` enters as ``pending / sqrt(mean(pending^2) + eps) * weight`` (32-bit; ``weight`` one number or ``hidden`` of them).
+    ``extra``: a 32-bit ``[T, hidden]`` tensor that the next norm adds to the residual too (an embedding that enters the stream again).
+    Only norms that say ``folds_post_norm`` know the two."""
+
+    __slots__ = ("residual", "pending", "normed", "fold", "post", "extra")
 
     def __init__(self, residual: torch.Tensor, pending: torch.Tensor | None = None):
         self.residual = residual
         self.pending = pending
         self.normed = None      # blocks whose norm follows the sum: the residual in the activation dtype, as the last norm left it
         self.fold = None
+        self.post = None
+        self.extra = None
 
 
 class LazyNorm:
@@ -301,7 +311,9 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    def paged_need(self) -> PagedNeed | None:
+    def paged_need(self) -> "PagedNeed | tuple[PagedNeed, ...] | None":
+        """One need, or several (each a group of pages with a block table of its own: ``cache.group`` / ``cache.planes`` are the first
+        one's, ``cache.more[i]`` the others')."""
         return None
 
     def state_need(self) -> StateNeed | None:

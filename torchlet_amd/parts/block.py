@@ -10,9 +10,13 @@ The other arrangement built here puts the norm after the sum: ``x <- norm1(alpha
 kernel that leaves the stream in 32-bit and, for the products that read it next, in the activation dtype.
 
 A third one keeps several copies of the residual, joined by hyper-connections (:class:`HyperConnectionBlock`).
+
+A fourth one norms a sublayer's output as well as its input (:class:`SandwichBlock`): ``x <- x + post1(mixer(norm1(x)))``, then ``x <- x +
+post2(ffn(norm2(x)))``; the output is left pending with its norm's weight, and the next norm's kernel norms it, adds it and norms the sum.
 """
 from __future__ import annotations
 
+from ..config.base import ConfigError
 from .base import BLOCKS, FEED_FORWARDS, KEEP_FLOAT32, MIXERS, NORMS, Block, Stream, WeightSpec, join_name, under
 
 
@@ -134,4 +138,40 @@ class HyperConnectionBlock(Block):
         if self.ffn is not None:
             h = self.ffn_norm.forward(stream, read=self.read[1])
             stream.pending, stream.fold = self.ffn.forward(h, ctx), self.fold[1]
+        return stream
+
+
+@BLOCKS.register("sandwich_residual")
+class SandwichBlock(Block):
+    """A norm before and after each sublayer.  The norm after a sublayer is not run here: its weight and eps are left on the stream
+    (``stream.post``) beside the pending output, and the next norm that folds the stream (this block's second one, the next block's first
+    one, the model's final one) does ``x += pending / rms(pending) * weight`` in 32-bit inside its own kernel.  So every norm that can follow
+    must be of a kind that says ``folds_post_norm``, and the norms after the sublayers must be root-mean-square norms with a plain weight."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.mixer_norm = NORMS.build(spec.mixer_norm, dtype, device)
+        self.mixer = MIXERS.build(spec.mixer, dtype, device)
+        self.mixer_post = NORMS.build(spec.mixer_post_norm, dtype, device)
+        self.ffn = FEED_FORWARDS.build(spec.ffn, dtype, device) if spec.ffn is not None else None
+        self.ffn_norm = NORMS.build(spec.ffn_norm, dtype, device) if spec.ffn is not None else None
+        self.ffn_post = NORMS.build(spec.ffn_post_norm, dtype, device) if spec.ffn is not None else None
+        self._children = {spec.mixer_norm_name: self.mixer_norm, spec.mixer_name: self.mixer, spec.mixer_post_norm_name: self.mixer_post}
+        if self.ffn is not None:
+            self._children.update({spec.ffn_norm_name: self.ffn_norm, spec.ffn_name: self.ffn, spec.ffn_post_norm_name: self.ffn_post})
+        for norm in (self.mixer_norm, self.mixer_post, self.ffn_norm, self.ffn_post):
+            if norm is not None and not getattr(norm, "folds_post_norm", False):
+                raise ConfigError(f"a block with norms after its sublayers needs norms that fold a normed branch output; {type(norm).__name__} does not")
+
+    parts = PreNormBlock.parts
+    weight_specs = PreNormBlock.weight_specs
+    load_weights = PreNormBlock.load_weights
+
+    def forward(self, stream: Stream, ctx, cache) -> Stream:
+        h = self.mixer_norm.forward(stream)
+        stream.pending, stream.post = self.mixer.forward(h, ctx, cache), (self.mixer_post.weight, self.mixer_post.eps)
+        if self.ffn is not None:
+            h = self.ffn_norm.forward(stream)
+            stream.pending, stream.post = self.ffn.forward(h, ctx), (self.ffn_post.weight, self.ffn_post.eps)
         return stream

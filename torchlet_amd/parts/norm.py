@@ -26,6 +26,11 @@ def _over_streams(kind: str, stream: Stream, weight, bias, eps: float, dtype, ro
     return out
 
 
+def _no_post_norm(stream: Stream, kind: str) -> None:
+    if stream.post is not None or stream.extra is not None:
+        raise ValueError(f"a {kind} does not fold a normed branch output or a second addend into the stream; a norm that says folds_post_norm does")
+
+
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
     graph_safe = True
@@ -43,6 +48,7 @@ class RMSNorm(Norm):
         self.weight = self._place(tensors[self.spec.weight_name], KEEP_STORED)
 
     def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0, read: torch.Tensor | None = None) -> torch.Tensor:
+        _no_post_norm(stream, "rmsnorm")
         if stream.residual.dim() == 3:
             return _over_streams("rmsnorm", stream, self.weight, None, self.eps, self.dtype, rows, gain, read)
         n = stream.residual.shape[0] if rows is None else rows.numel()
@@ -91,4 +97,38 @@ class LayerNorm(Norm):
         self.bias = self._place(tensors[self.spec.bias_name], KEEP_FLOAT32)
 
     def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0, read: torch.Tensor | None = None) -> torch.Tensor:
+        _no_post_norm(stream, "layernorm")
         return _over_streams("layernorm", stream, self.weight, self.bias, self.eps, self.dtype, rows, gain, read)
+
+
+@NORMS.register("scalar_rmsnorm")
+class ScalarRMSNorm(Norm):
+    """``r / sqrt(mean(r^2) + eps) * g`` with one number ``g`` for all coordinates, in 32-bit.  It folds everything a stream can carry
+    into the residual on the way, in the same kernel: the pending branch output, plain or, where the block left a norm on it
+    (``stream.post``), divided by its own root mean square and multiplied by that norm's weight first; and a second addend
+    (``stream.extra``)."""
+    graph_safe = True
+    folds_post_norm = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.dim = spec.dim
+        self.eps = float(spec.eps)
+        self.weight: torch.Tensor | None = None
+
+    def weight_specs(self):
+        return {self.spec.weight_name: WeightSpec((), keep=KEEP_FLOAT32, init="one_plus_normal")}
+
+    def load_weights(self, tensors):
+        self.weight = self._place(tensors[self.spec.weight_name].reshape(1), KEEP_FLOAT32)
+
+    def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0, read: torch.Tensor | None = None) -> torch.Tensor:
+        if stream.residual.dim() != 2 or stream.fold is not None:
+            raise ValueError("a scalar_rmsnorm runs over one plain residual")
+        n = stream.residual.shape[0] if rows is None else rows.numel()
+        out = torch.empty((n, self.dim), dtype=self.dtype, device=stream.residual.device)
+        post_w, post_eps = stream.post if stream.post is not None else (None, 0.0)
+        ops.sandwich_norm(stream.residual, stream.pending, post_w, post_eps, stream.extra, self.weight, self.eps, out, rows, gain)
+        if rows is None:
+            stream.pending = stream.post = stream.extra = None
+        return out

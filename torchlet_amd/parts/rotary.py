@@ -54,8 +54,9 @@ class PairRotaryEncoding(PositionEncoding):
         if spec.dims % 2 or spec.dims <= 0:
             raise ConfigError(f"rotary encoding in pairs needs an even, positive number of dimensions, got {spec.dims}")
         self.dims = spec.dims
+        self.halves = False
         i = torch.arange(spec.dims // 2, dtype=torch.float64)
-        self.inv_freq = (float(spec.base) ** (-2.0 * i / spec.dims)).to(torch.float32).to(device)
+        self.inv_freq = (float(spec.base) ** (-2.0 * i / spec.dims) / float(getattr(spec, "factor", 1.0))).to(torch.float32).to(device)
 
     def apply(self, q, k, positions):
         for x in (q, k):
@@ -64,3 +65,31 @@ class PairRotaryEncoding(PositionEncoding):
             T, heads, hd = x.shape
             flat = x.as_strided((T, heads * hd), (x.stride(0), 1))
             ops.rotate_pairs(flat, hd, 0, flat, hd, 0, positions, self.inv_freq, heads, hd)
+
+
+@POSITION_ENCODINGS.register("rope_halves")
+class HalfRotaryEncoding(PositionEncoding):
+    """The rotate-half layout over the first ``dims`` entries of a vector: entry ``i`` is paired with ``i + dims / 2`` and the pair
+    ``(u, v)`` at position ``p`` becomes ``(u cos a - v sin a, v cos a + u sin a)`` with ``a = float32(p) * f_i``, ``f_i = base**(-2i / dims) /
+    factor`` (taken in 64-bit on the host, then rounded once to 32-bit); entries beyond ``dims`` pass unchanged.  Mixers fold the rotation
+    into their own kernels through :attr:`inv_freq`, :attr:`dims` and :attr:`halves`; :meth:`apply` turns whole heads in place."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        if spec.dims % 2 or spec.dims <= 0:
+            raise ConfigError(f"rotary encoding over halves needs an even, positive number of dimensions, got {spec.dims}")
+        if not float(spec.factor) > 0:
+            raise ConfigError(f"rotary encoding: the scaling factor must be positive, got {spec.factor}")
+        self.dims = spec.dims
+        self.halves = True
+        i = torch.arange(spec.dims // 2, dtype=torch.float64)
+        self.inv_freq = (float(spec.base) ** (-2.0 * i / spec.dims) / float(spec.factor)).to(torch.float32).to(device)
+
+    def apply(self, q, k, positions):
+        for x in (q, k):
+            if x is None:
+                continue
+            T, heads, hd = x.shape
+            flat = x.as_strided((T, heads * hd), (x.stride(0), 1))
+            ops.head_norm_rotate(flat, heads, 0, hd, None, None, 0.0, positions, self.inv_freq, self.dims, True)

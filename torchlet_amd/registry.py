@@ -9,6 +9,7 @@ import json
 from pathlib import Path
 
 from .config.base import ConfigError, ModelConfig
+from .config.fotovik import FotovikConfig
 from .config.migurax import MiguraxConfig
 from .config.nebutar import NebutarConfig
 from .config.qwen2 import Qwen2Config
@@ -30,6 +31,7 @@ def unregister_architecture(name: str) -> None:
 register_architecture(Qwen2Config)
 register_architecture(MiguraxConfig)
 register_architecture(NebutarConfig)
+register_architecture(FotovikConfig)
 
 
 def config_class(name: str) -> type[ModelConfig]:
