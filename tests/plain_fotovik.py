@@ -198,8 +198,9 @@ def run_order(config):
     return order + [(i, False) for i in range(b, n)]
 
 
-def forward(config, w, tokens, cached=lambda x: x):
-    """``(logits [T, vocab], residual after every layer run [runs, T, width])``, 64-bit."""
+def forward(config, w, tokens, cached=lambda x: x, stored=lambda x: x):
+    """``(logits [T, vocab], residual after every layer run [runs, T, width])``, 64-bit.  ``stored``: a rounding of what the sublayers read
+    and hand back (to see what an engine that keeps those in fewer bits may differ by); ``cached``: the same for cached keys and values."""
     eps = float(config["norm"]["eps"])
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     x0 = embedding(config, w, tokens)
@@ -209,11 +210,11 @@ def forward(config, w, tokens, cached=lambda x: x):
         layer, name = config["layers"][i], f"l{i}."
         if again:
             x = x + x0
-        y = mixer(layer, w, name + "mix.", rms(x, eps) * w[name + "norm1"].to(F64), eps, cached)
+        y = stored(mixer(layer, w, name + "mix.", stored(rms(x, eps) * w[name + "norm1"].to(F64)), eps, cached))
         x = x + rms(y, eps) * w[name + "norm1b"].to(F64)
         if layer.get("mlp"):
-            y = dense_ff(w, name + "mlp.", rms(x, eps) * w[name + "norm2"].to(F64))
+            y = stored(dense_ff(w, name + "mlp.", stored(rms(x, eps) * w[name + "norm2"].to(F64))))
             x = x + rms(y, eps) * w[name + "norm2b"].to(F64)
         after.append(x.clone())
-    logits = (rms(x, eps) * w["final.norm"].to(F64)) @ w["head"].to(F64).T
+    logits = stored(rms(x, eps) * w["final.norm"].to(F64)) @ w["head"].to(F64).T
     return logits, torch.stack(after)
