@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16]
                     [--shape 7b|14b|32b] [--context N] [--new-tokens G] [--prefill-tokens T]
-                    [--workload decode|serve|migurax|nebutar] [--only decode|step|prefill] [--all]
+                    [--workload decode|serve|migurax|nebutar|fotovik] [--only decode|step|prefill] [--all]
 
 The default run has the layer sizes of Qwen2.5-7B (28 layers, hidden 3584, 28 heads, 4 KV heads, head
 size 128, intermediate 18944, vocabulary 152064) with random weights and goes through the whole engine
@@ -44,6 +44,11 @@ the bytes it must move or the operations it must do and the fraction of the GPU'
 with soft-capped scores in chunks beside a gated delta rule; gated experts, some of them the identity), beside the Migurax model of
 the same width and layer count (the closest one the framework has: a recurrent state per request and routed experts), and its own
 kernels beside the like kernels of the Migurax and Qwen2 paths.
+
+``--workload fotovik [--size s|m]`` does the same for the Fotovik design (a norm before and after every sublayer; attention with a window,
+pooled blocks before it and a sink; causal attention with normed queries and keys beside linear attention with fixed decays; a gated
+delta rule; dense feed-forwards), beside the Nebutar model of the same width and layer count (the closest one the framework has: two
+mixers side by side, a delta rule, a span of layers, the same attention kernels), and its own kernels beside their like.
 """
 from __future__ import annotations
 
@@ -86,8 +91,8 @@ def parse_args(argv=None):
     p.add_argument("--context", type=int, default=CONTEXT, help="prompt tokens of each request in the decode runs")
     p.add_argument("--new-tokens", type=int, default=None, help="tokens each request may generate (decode: 256, serve: 128)")
     p.add_argument("--prefill-tokens", type=int, default=2048)
-    p.add_argument("--workload", choices=["decode", "serve", "migurax", "nebutar"], default="decode")
-    p.add_argument("--size", choices=["s", "m"], default="s", help="migurax, nebutar: layer sizes (s: width 2048, m: width 4096)")
+    p.add_argument("--workload", choices=["decode", "serve", "migurax", "nebutar", "fotovik"], default="decode")
+    p.add_argument("--size", choices=["s", "m"], default="s", help="migurax, nebutar, fotovik: layer sizes (s: width 2048, m: width 4096)")
     p.add_argument("--requests", type=int, default=32)
     p.add_argument("--prompt-min", type=int, default=128)
     p.add_argument("--prompt-max", type=int, default=4096)
@@ -900,6 +905,183 @@ def nebutar(args) -> dict:
         out["kernels"] = nebutar_kernels(ours, like, args.batch, args.context, args.prefill_tokens)
     return out
 
+# ---------------------------------------------------------------------------------------------- the Fotovik design
+
+def fotovik_sizes(size: str) -> dict:
+    """A Fotovik configuration of four layers (the middle two form a span that runs once) at the width of the other designs' sizes: causal
+    attention with heads of 128 + 128 beside linear attention with heads of 128 x 128; attention in a window of 1024 with blocks of 64 before
+    it; a delta rule with heads of 128 x 128 behind convolutions of four taps; dense feed-forwards of four times the width."""
+    width, heads = dict(s=(2048, 16), m=(4096, 32))[size]
+    rot = dict(dims=64, base=1000000.0)
+    left = dict(heads=heads, kv_heads=heads // 4, dim=128, vdim=128, scale=128 ** -0.5, rot=dict(rot, scaling=dict(factor=2.0)))
+    right = dict(heads=heads, dim=128, vdim=128, decay=[1.0 - 2.0 ** -(3 + 5 * i / max(1, heads - 1)) for i in range(heads)])
+    windowed = dict(heads=heads, kv_heads=heads // 4, dim=128, vdim=128, scale=128 ** -0.5, rot=rot, mask=dict(size=1024, pool=64))
+    delta = dict(heads=heads, kv_heads=heads // 2, dim=128, vdim=128, conv=4)
+    mlp = dict(kind="dense", ff=4 * width)
+    return dict(architecture="Fotovik", vocab=32000, width=width, max_positions=8192, norm=dict(eps=1e-5),
+                embedding=dict(scale=1.0, bigram=dict(buckets=65521, mul_prev=36313, mul_cur=27191)), loop=dict(start=1, stop=3, times=1),
+                layers=[dict(type="parallel", mixer=dict(left=left, right=right), mlp=mlp), dict(type="attention", mixer=windowed, mlp=mlp),
+                        dict(type="delta", mixer=delta, mlp=mlp), dict(type="attention", mixer=windowed, mlp=mlp)])
+
+
+def fotovik_kernels(ours: dict, like: dict, batch: int, context: int, tokens: int) -> list[dict]:
+    """Each kernel that is the design's own, alone, at the sizes of ``ours``, in a decode step of ``batch`` requests on ``context`` cached
+    tokens and in a prompt of ``tokens`` tokens, beside the like kernel of the Nebutar or Qwen2 path.  ``frac``: bytes that must move / time
+    against 8 TB/s, or operations / time against the matrix cores' bfloat16 rate (against the 32-bit rate for the recurrences)."""
+    import torch
+    from torchlet_amd.kernels import ops
+    dev, bf = "cuda", torch.bfloat16
+    rows = []
+
+    def add(name, kind, launch, nbytes=0.0, flops=0.0, peak=MFMA_PEAK_TFLOPS["bfloat16"]):
+        ms = _best_ms(launch, rounds=3, calls=5)
+        row = {"kernel": name, "like": kind, "ms": round(ms, 4)}
+        if nbytes:
+            row.update(bytes=int(nbytes), frac=round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), bound="hbm")
+        else:
+            row.update(flops=flops, frac=round(flops / (ms * 1e-3) / (peak * 1e12), 4), bound="flops")
+        rows.append(row)
+        say(f"  {name}: {ms:.4f} ms, {row['frac']} of its bound")
+
+    def tables(n_req, total, span=PAGE):
+        blocks = -(-total // span)
+        table = (torch.arange(n_req * blocks, dtype=torch.int32, device=dev) + 1).view(n_req, blocks)
+        return table, n_req * blocks + 1
+
+    width = ours["width"]
+    par, att, delta = ours["layers"][0]["mixer"], ours["layers"][1]["mixer"], ours["layers"][2]["mixer"]
+    # ---- linear attention with fixed decays beside the delta rule (the same kernel without the correction): a decode step reads and writes
+    #      every state once; a prompt does 4 operations per state element and token (the update and one sum over the rows), the delta rule 6
+    lin = par["right"]
+    h, d, v = lin["heads"], lin["dim"], lin["vdim"]
+    dh, dg, dd, dv_ = delta["heads"], delta["kv_heads"], delta["dim"], delta["vdim"]
+    for name, T, reqs in (("decay_scan decode", batch, batch), (f"decay_scan prompt {tokens}", tokens, 1)):
+        qkv = torch.randn(T, 2 * h * d + h * v, device=dev) * 0.1
+        decay = torch.tensor(lin["decay"], device=dev)
+        state = torch.zeros(reqs + 1, h * d * v, device=dev)
+        out = torch.empty(T, h * v, device=dev)
+        slots = torch.arange(reqs, dtype=torch.int32, device=dev)
+        indptr = (torch.arange(reqs + 1, dtype=torch.int32, device=dev) * (T // reqs))
+        launch = lambda: ops.decay_scan(qkv, decay, state, slots, indptr, out, h, d, v, max_new_tokens=T // reqs)
+        if reqs > 1:
+            add(name, "delta_scan decode", launch, nbytes=2.0 * reqs * h * d * v * 4)
+        else:
+            add(name, f"delta_scan prompt {tokens}", launch, flops=4.0 * T * h * d * v, peak=MFMA_PEAK_TFLOPS["float32"])
+        qkv2 = torch.randn(T, 2 * dg * dd + dh * dv_, device=dev) * 0.1
+        gates = torch.rand(T, 2 * dh, device=dev) * 0.5 + 0.5
+        state2 = torch.zeros(reqs + 1, dh * dd * dv_, device=dev)
+        out2 = torch.empty(T, dh * dv_, device=dev)
+        launch = lambda: ops.delta_scan(qkv2, gates, state2, slots, indptr, out2, dh, dg, dd, dv_, max_new_tokens=T // reqs)
+        if reqs > 1:
+            add(name.replace("decay_scan", "delta_scan") + " (the design's own delta layers, and the Nebutar path)", "", launch, nbytes=2.0 * reqs * dh * dd * dv_ * 4)
+        else:
+            add(name.replace("decay_scan", "delta_scan") + " (the design's own delta layers, and the Nebutar path)", "", launch,
+                flops=6.0 * T * dh * dd * dv_, peak=MFMA_PEAK_TFLOPS["float32"])
+    # ---- attention in a window with pooled blocks and a sink, and causal attention, beside the Nebutar path's attention in chunks (the
+    #      same kernels): a decode step reads the keys and values it may see once; a prompt's scores and sums
+    nb = like["layers"][0]["mixer"]["left"]
+    for label, m, window, pool, chunk, cap, sink_on in (("window 1024, blocks of 64, sink", att, att["mask"]["size"], att["mask"]["pool"], 0, 0.0, True),
+                                                        ("causal", par["left"], 0, 0, 0, 0.0, False),
+                                                        ("chunks of 1024, capped (Nebutar path)", nb, 0, 0, nb["mask"]["size"], nb["softcap"], False)):
+        H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        for T, reqs, ctx in ((batch, batch, context - 1), (tokens, 1, 0)):
+            total = ctx + T // reqs
+            table, pages = tables(reqs, total)
+            k_plane = (torch.randn(pages, G, PAGE, dk, device=dev) * 0.3).to(bf)
+            v_plane = (torch.randn(pages, G, dv, PAGE, device=dev) * 0.3).to(bf)
+            pooled = None
+            if pool:
+                ptable, ppages = tables(reqs, total, PAGE * pool)
+                ptable = torch.nn.functional.pad(ptable, (0, table.shape[1] - ptable.shape[1])).contiguous()
+                pooled = ((torch.randn(ppages, G, PAGE, dk, device=dev) * 0.3).to(bf), (torch.randn(ppages, G, dv, PAGE, device=dev) * 0.3).to(bf), ptable, pool)
+            sink = torch.zeros(H, device=dev) if sink_on else None
+            q = (torch.randn(T, H * dk, device=dev) * 0.3).to(bf)
+            out = torch.empty(T, H * dv, dtype=bf, device=dev)
+            token_req = torch.arange(T, dtype=torch.int32, device=dev) // (T // reqs)
+            positions = (torch.arange(T, dtype=torch.int32, device=dev) % (T // reqs)) + ctx
+            if reqs == 1:
+                n_tiles = -(-T // ops.LOCAL_ATTENTION_TILE_TOKENS)
+                tiles = (torch.tensor([0, T], dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int32, device=dev),
+                         torch.zeros(n_tiles, dtype=torch.int32, device=dev), torch.arange(n_tiles, dtype=torch.int32, device=dev) * ops.LOCAL_ATTENTION_TILE_TOKENS, n_tiles)
+            else:
+                tiles = (torch.arange(reqs + 1, dtype=torch.int32, device=dev), torch.full((reqs,), ctx, dtype=torch.int32, device=dev), None, None, reqs)
+            launch = lambda: ops.local_attention(q, out, k_plane, v_plane, table, token_req, positions, H, G, dk, dv, PAGE, m["scale"], cap, chunk, window, 1.0,
+                                                 tiles=tiles, sink=sink, pooled=pooled)
+
+            def seen(p):        # keys (tokens and pooled rows) that a query at position p reads
+                lo = max(p // chunk * chunk if chunk else 0, p - window + 1 if window else 0)
+                return p - lo + 1 + (max(0, p - window + 1) // pool if pool else 0)
+            if reqs > 1:
+                add(f"local_attention decode, {label}", "local_attention decode, chunks", launch, nbytes=float(reqs) * seen(ctx) * G * (dk + dv) * 2)
+            else:
+                add(f"local_attention prompt {tokens}, {label}", f"local_attention prompt {tokens}, chunks", launch,
+                    flops=2.0 * H * (dk + dv) * sum(seen(p) for p in range(T)))
+    # ---- the norm that norms what it adds beside the plain residual's norm: reads the residual and the branch output, writes residual and row
+    for name, T in (("sandwich_norm decode", batch), (f"sandwich_norm prompt {tokens}", tokens)):
+        res = torch.randn(T, width, device=dev)
+        pen = torch.randn(T, width, device=dev).to(bf)
+        one = torch.ones(1, device=dev)
+        out = torch.empty(T, width, dtype=bf, device=dev)
+        add(name, "add_rmsnorm", lambda: ops.sandwich_norm(res, pen, one, 1e-5, None, one, 1e-5, out), nbytes=float(T) * width * 12)
+        wb = torch.ones(width, dtype=bf, device=dev)
+        add(name.replace("sandwich_norm", "add_rmsnorm") + " (Qwen2 path)", "", lambda: ops.add_rmsnorm(res, pen, wb, 1e-5, out), nbytes=float(T) * width * 12)
+    # ---- norm per head and rotation in place, the pooled rows of a prompt, the sum of the two normed branches, the embedding with its bigram row
+    H, G, dk = par["left"]["heads"], par["left"]["kv_heads"], par["left"]["dim"]
+    T = tokens
+    x = torch.randn(T, (H + 2 * G) * dk, device=dev).to(bf)
+    wq = torch.ones(dk, device=dev)
+    positions = torch.arange(T, dtype=torch.int32, device=dev)
+    inv = torch.rand(32, device=dev)
+    add(f"head_norm_rotate prompt {tokens}", "rope_cache_write", lambda: ops.head_norm_rotate(x[:, : (H + G) * dk], H, G, dk, wq, wq, 1e-5, positions, inv, 64, True),
+        nbytes=float(T) * (H + G) * dk * 4)
+    G, dk, dv, pool = att["kv_heads"], att["dim"], att["vdim"], att["mask"]["pool"]
+    table, pages = tables(1, T)
+    ptable, ppages = tables(1, T, PAGE * pool)
+    k_plane, v_plane = torch.randn(pages, G, PAGE, dk, device=dev).to(bf), torch.randn(pages, G, dv, PAGE, device=dev).to(bf)
+    pk, pv = torch.zeros(ppages, G, PAGE, dk, dtype=bf, device=dev), torch.zeros(ppages, G, dv, PAGE, dtype=bf, device=dev)
+    indptr, zero = torch.tensor([0, T], dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int32, device=dev)
+    add(f"pool_blocks prompt {tokens}", "kv_cache_write", lambda: ops.pool_blocks(k_plane, v_plane, table, pk, pv, ptable, indptr, zero, T // pool + 1, PAGE, pool),
+        nbytes=float(T) * G * (dk + dv) * 2)
+    outs = torch.randn(2, T, width, device=dev).to(bf)
+    w2 = torch.ones(2, width, device=dev)
+    y = torch.empty(T, width, dtype=bf, device=dev)
+    add(f"normed_sum prompt {tokens}", "add_rmsnorm", lambda: ops.normed_sum(outs, w2, 1e-5, y), nbytes=float(T) * width * 6)
+    big = ours["embedding"]["bigram"]
+    emb, bigram = torch.randn(ours["vocab"], width, device=dev).to(bf), torch.randn(big["buckets"] + 1, width, device=dev).to(bf)
+    ids = torch.randint(0, ours["vocab"], (T,), dtype=torch.int32, device=dev)
+    res2 = torch.empty(T, width, device=dev)
+    last = torch.zeros(2, 1, dtype=torch.int32, device=dev)
+    token_req = torch.zeros(T, dtype=torch.int32, device=dev)
+    add(f"bigram_embedding prompt {tokens}", "embedding", lambda: ops.bigram_embedding(ids, emb, res2, 1.0, bigram, big["buckets"], big["mul_prev"], big["mul_cur"],
+                                                                                     token_req, indptr, positions, zero, last), nbytes=float(T) * width * 8)
+    add(f"embedding prompt {tokens} (Qwen2 path)", "", lambda: ops.embedding(ids, emb, res2, 1.0), nbytes=float(T) * width * 6)
+    return rows
+
+
+def fotovik(args) -> dict:
+    import torch
+    ours = fotovik_sizes(args.size)
+    like = nebutar_sizes(args.size)
+    out = {"metric": f"Fotovik design, size {args.size} (width {ours['width']}, 4 layers), prefill of {args.prefill_tokens} tokens and decode at batch "
+                     f"{args.batch} on {args.context}-token caches, beside the Nebutar design at equal width and layer count, one MI355X",
+           "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+           "data": "synthetic: seeded random weights, token ids and cache contents", "config": {"fotovik": ours, "nebutar": like}}
+    for key, d in (("fotovik", ours), ("nebutar", like)):
+        say(f"building the {key} model")
+        cfg, model = _build_from(d, args.dtype)
+        pms, pbest = time_prefill(model, args.prefill_tokens)
+        dms = _decode_ms(model, args.batch, min(args.steps, 64), args.warmup, args.context)
+        out[key] = {"weight_bytes": _weight_bytes(model),
+                    "prefill": {"tokens": args.prefill_tokens, "ms": round(pms, 3), "ms_best": round(pbest, 3), "tokens_per_s": round(args.prefill_tokens * 1e3 / pms, 1)},
+                    "decode": {"batch": args.batch, "context": args.context, "ms_per_step": round(dms, 4), "tokens_per_s": round(args.batch * 1e3 / dms, 1)}}
+        say(f"{key}: {out[key]}")
+        del model
+        torch.cuda.empty_cache()
+    out["value"] = out["fotovik"]["decode"]["tokens_per_s"]
+    if args.dtype == "bfloat16" and not args.no_points:
+        out["kernels"] = fotovik_kernels(ours, like, args.batch, args.context, args.prefill_tokens)
+    return out
+
 
 def main(argv=None) -> int:
     args = parse_args(argv)
@@ -917,6 +1099,9 @@ def main(argv=None) -> int:
         return 0
     if args.workload == "nebutar":
         print(json.dumps(nebutar(args)))
+        return 0
+    if args.workload == "fotovik":
+        print(json.dumps(fotovik(args)))
         return 0
     name, sizes = SHAPES[args.shape]
     full_layers = sizes["num_hidden_layers"]
