@@ -1042,6 +1042,9 @@ def fotovik_kernels(ours: dict, like: dict, batch: int, context: int, tokens: in
     indptr, zero = torch.tensor([0, T], dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int32, device=dev)
     add(f"pool_blocks prompt {tokens}", "kv_cache_write", lambda: ops.pool_blocks(k_plane, v_plane, table, pk, pv, ptable, indptr, zero, T // pool + 1, PAGE, pool),
         nbytes=float(T) * G * (dk + dv) * 2)
+    kk, vv = torch.randn(T, G * dk, device=dev).to(bf), torch.randn(T, G * dv, device=dev).to(bf)
+    add(f"kv_cache_write prompt {tokens} (Nebutar path)", "", lambda: ops.kv_cache_write(kk, vv, torch.zeros(T, dtype=torch.int32, device=dev), positions, table, k_plane, v_plane, PAGE),
+        nbytes=float(T) * G * (dk + dv) * 4)
     outs = torch.randn(2, T, width, device=dev).to(bf)
     w2 = torch.ones(2, width, device=dev)
     y = torch.empty(T, width, dtype=bf, device=dev)

@@ -465,13 +465,15 @@ extern "C" int tl_local_attention(const void* q, int q_ld, void* out, int out_ld
 // ------------------------------------------------------------------ pooled blocks
 // Block b of a request (positions b * pool .. b * pool + pool - 1) gets its pooled key and value, the means of its cached keys and values,
 // in the step that brings its last token: the blocks ctx / pool .. (ctx + n) / pool - 1 of a request that held ctx tokens and gets n.  One
-// work-group per such block; sums in float in the order of the positions, one rounding.  Pooled rows lie in planes laid out like the
-// tokens' (values transposed) under a block table of their own, block b in row b; what would go to page 0 is dropped.
+// wave per such block, key/value head and 64 columns of keys-and-values side by side (a lane owns a column and walks the block's
+// positions); sums in float in the order of the positions, one rounding.  Pooled rows lie in planes laid out like the tokens' (values
+// transposed) under a block table of their own, block b in row b; what would go to page 0 is dropped.
 template <typename T>
-__global__ void pool_blocks_kernel(const T* __restrict__ k_plane, const T* __restrict__ v_plane, const int* __restrict__ block_table, int table_ld,
-                                   int table_width, T* __restrict__ pk_plane, T* __restrict__ pv_plane, const int* __restrict__ pool_table,
-                                   int pool_table_ld, int pool_table_width, const int* __restrict__ req_indptr, const int* __restrict__ ctx_lens,
-                                   int kv_heads, int dim, int vdim, int pages, int pool_pages, int page_size, int pool) {
+__global__ void __launch_bounds__(TL_WAVE)
+pool_blocks_kernel(const T* __restrict__ k_plane, const T* __restrict__ v_plane, const int* __restrict__ block_table, int table_ld,
+                   int table_width, T* __restrict__ pk_plane, T* __restrict__ pv_plane, const int* __restrict__ pool_table,
+                   int pool_table_ld, int pool_table_width, const int* __restrict__ req_indptr, const int* __restrict__ ctx_lens,
+                   int kv_heads, int dim, int vdim, int pages, int pool_pages, int page_size, int pool) {
     const int r = blockIdx.y;
     const int ctx = ctx_lens[r], n = req_indptr[r + 1] - req_indptr[r];
     const int b = ctx / pool + blockIdx.x;
@@ -482,23 +484,22 @@ __global__ void pool_blocks_kernel(const T* __restrict__ k_plane, const T* __res
     if (ppage <= 0 || ppage >= pool_pages) return;
     const int pslot = b % page_size;
     const int* table = block_table + (size_t)r * table_ld;
-    const float inv = 1.f / (float)pool;
-    for (int i = threadIdx.x; i < kv_heads * (dim + vdim); i += blockDim.x) {
-        const bool is_key = i < kv_heads * dim;
-        const int e = is_key ? i : i - kv_heads * dim;
-        const int width = is_key ? dim : vdim;
-        const int g = e / width, d = e % width;
-        float sum = 0.f;
-        for (int j = 0; j < pool; ++j) {
-            const int key = b * pool + j, blk = key / page_size, slot = key % page_size;
-            const int page = blk < table_width ? table[blk] : 0;
-            if (page <= 0 || page >= pages) continue;          // (a block's tokens are all held when its last one arrives)
-            sum += is_key ? to_float(k_plane[(((size_t)page * kv_heads + g) * page_size + slot) * dim + d])
-                          : to_float(v_plane[(((size_t)page * kv_heads + g) * vdim + d) * page_size + slot]);
-        }
-        if (is_key) pk_plane[(((size_t)ppage * kv_heads + g) * page_size + pslot) * dim + d] = from_float<T>(sum * inv);
-        else pv_plane[(((size_t)ppage * kv_heads + g) * vdim + d) * page_size + pslot] = from_float<T>(sum * inv);
+    const int chunks = (dim + vdim + TL_WAVE - 1) / TL_WAVE;
+    const int g = blockIdx.z / chunks, e = (blockIdx.z % chunks) * TL_WAVE + threadIdx.x;
+    if (e >= dim + vdim) return;
+    const bool is_key = e < dim;
+    const int d = is_key ? e : e - dim;
+    float sum = 0.f;
+    for (int j = 0; j < pool; ++j) {
+        const int key = b * pool + j, blk = key / page_size, slot = key % page_size;
+        const int page = blk < table_width ? table[blk] : 0;
+        if (page <= 0 || page >= pages) continue;          // (a block's tokens are all held when its last one arrives)
+        sum += is_key ? to_float(k_plane[(((size_t)page * kv_heads + g) * page_size + slot) * dim + d])
+                      : to_float(v_plane[(((size_t)page * kv_heads + g) * vdim + d) * page_size + slot]);
     }
+    const float mean = sum / (float)pool;
+    if (is_key) pk_plane[(((size_t)ppage * kv_heads + g) * page_size + pslot) * dim + d] = from_float<T>(mean);
+    else pv_plane[(((size_t)ppage * kv_heads + g) * vdim + d) * page_size + pslot] = from_float<T>(mean);
 }
 
 // `most_blocks`: an upper bound of the blocks one request completes in the step (its longest portion / pool + 1).
@@ -510,7 +511,9 @@ extern "C" int tl_pool_blocks(const void* k_plane, const void* v_plane, int page
                "pool_blocks: bad sizes");
     TL_REQUIRE(table_ld >= table_width && pool_table_ld >= pool_table_width && table_width > 0 && pool_table_width > 0, "pool_blocks: block tables too short");
     if (requests == 0 || most_blocks == 0) return TL_OK;
-    dim3 grid(most_blocks, requests), block(256);
+    const int chunks = (dim + vdim + TL_WAVE - 1) / TL_WAVE;
+    TL_REQUIRE((long)kv_heads * chunks <= 65535, "pool_blocks: too many heads");
+    dim3 grid(most_blocks, requests, kv_heads * chunks), block(TL_WAVE);
     if (dtype == TL_DT_F32)
         pool_blocks_kernel<float><<<grid, block, 0, stream>>>((const float*)k_plane, (const float*)v_plane, (const int*)block_table, table_ld, table_width,
             (float*)pk_plane, (float*)pv_plane, (const int*)pool_table, pool_table_ld, pool_table_width, (const int*)req_indptr, (const int*)ctx_lens,
