@@ -144,6 +144,32 @@ def test_step_function_equals_plain_under_every_split(cpu_ops, folders, name, mo
     assert runner.cache.live_requests() == [] and runner.cache.free_pages() == runner.cache.capacity()
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_configurations_drawn_at_random(cpu_ops, tmp_path, seed):
+    """Layers of any kind in any order and any span of them run again, through the host side: portions and mixed batches against plain."""
+    import random
+    rnd = random.Random(700 + seed)
+    conf = tiny_fotovik.random_config(rnd, big=False)
+    page = rnd.choice([4, 8, 16])
+    folder = tiny_fotovik.write(f"random{seed}", tmp_path, config=conf, seed=seed)
+    w = {k: v.double() for k, v in tiny_fotovik.tensors_for("", 1.0, conf, seed).items()}
+    seqs, refs = tiny_fotovik.sequences("", w, [rnd.randint(1, 60) for _ in range(4)], seed=seed, config=conf)
+    _, model = load_model(folder, "float32", device="cpu")
+    for mode in ("portions", "mixed"):
+        steps = scenarios.number(getattr(scenarios, mode)(seqs))
+        runner = make_runner(model, page_size=page, num_pages=-(-scenarios.max_tokens_needed(steps, unit=page) // page) + 1, max_requests=4)
+        out = {}
+        for s in steps:
+            logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+            if logits is not None:
+                out[s["step"]] = logits.numpy()
+            for r in s["end"]:
+                runner.release(r)
+            runner.cache.check()
+        scenarios.check(steps, out, refs, TOL, f"{conf}/{mode}")
+        assert runner.cache.free_pages() == runner.cache.capacity()
+
+
 def test_stream_after_every_layer_run_against_plain(cpu_ops, folders):
     """The residual after every run of a layer (a looped layer counts each time; the embedding that enters again counts with the run
     it comes before)."""

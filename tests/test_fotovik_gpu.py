@@ -163,6 +163,31 @@ def test_decode_steps_replayed_as_graphs(folders, dtype):
         torch.testing.assert_close(got[True][r], got[False][r], atol=tol["atol"] / 2, rtol=0.0)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Layers of any kind in any order, any span of them run again, sizes of the matrix-core kernels (even seeds) or small odd ones:
+    whole requests, portions and mixed batches in both dtypes against the plain implementation, every pool full at the end."""
+    import random
+    from torchlet_amd.engine.loading import load_model, make_runner
+    rnd = random.Random(500 + seed)
+    conf = tiny_fotovik.random_config(rnd, big=seed % 2 == 0)
+    page = 16 if seed % 2 == 0 else rnd.choice([4, 8, 16])
+    folder = tiny_fotovik.write(f"random{seed}", tmp_path, config=conf, seed=seed)
+    w = {k: v.double() for k, v in tiny_fotovik.tensors_for("", 1.0, conf, seed).items()}
+    seqs, refs = tiny_fotovik.sequences("", w, [rnd.randint(1, 120) for _ in range(4)], seed=seed, config=conf)
+    rounded = lambda t: t.to(torch.bfloat16).double()
+    for dtype in DTYPES:
+        tol = dict(atol=8e-4, rtol=3e-4)
+        if dtype == "bfloat16":
+            tol = dict(atol=3 * max(float((plain_fotovik.forward(conf, w, t, cached=rounded, stored=rounded)[0] - refs[r]).abs().max()) for r, t in seqs.items()), rtol=0.0)
+        _, model = load_model(folder, dtype)
+        for mode in ("whole", "portions", "mixed"):
+            steps = scenarios.number(getattr(scenarios, mode)(seqs))
+            runner = make_runner(model, page_size=page, num_pages=-(-scenarios.max_tokens_needed(steps, unit=page) // page) + 1, max_requests=4)
+            scenarios.check(steps, _replay(runner, steps), refs, tol, f"{conf}/{mode}/{dtype}")
+            assert runner.cache.live_requests() == [] and runner.cache.free_pages() == runner.cache.capacity()
+
+
 SHARP = dict(architecture="Fotovik", vocab=80, width=64, norm=dict(eps=1e-5), embedding=dict(scale=3.0, bigram=dict(buckets=41, mul_prev=9, mul_cur=4)), layers=[
     dict(type="attention", mixer=dict(heads=4, kv_heads=1, dim=32, vdim=32, scale=0.3, rot=dict(dims=8, base=10000.0), mask=dict(size=32, pool=8)),
          mlp=dict(kind="dense", ff=64)),

@@ -118,3 +118,47 @@ def sequences(name: str, weights, lengths, seed: int = 0, config: dict | None = 
     g = torch.Generator().manual_seed(seed)
     seqs = {f"r{i}": torch.randint(0, cfg["vocab"], (n,), generator=g).tolist() for i, n in enumerate(lengths)}
     return seqs, {r: plain_fotovik.forward(cfg, weights, t)[0] for r, t in seqs.items()}
+
+
+def _random_attention(rnd, big, with_mask):
+    if big:
+        dim, vdim = rnd.choice([32, 64, 96, 128]), rnd.choice([16, 32, 64, 128])
+    else:
+        dim, vdim = rnd.choice([4, 6, 10, 24]), rnd.choice([3, 8, 12])
+    kv_heads = rnd.choice([1, 2, 3])
+    m = _attention(kv_heads * rnd.choice([1, 2, 4]), kv_heads, dim, vdim, rnd.choice([0.1, 0.25, dim ** -0.5]))
+    if rnd.random() < 0.85:
+        m["rot"] = _rot(rnd.choice([d for d in (2, 4, 8, 16, 32, 64, 128) if d <= dim]), rnd.choice([100.0, 10000.0, 1e6]),
+                        rnd.choice([None, 1.0, 2.0, 8.0]))
+    if with_mask:
+        m["mask"] = dict(size=rnd.choice([1, 3, 7, 16, 33, 50]), pool=rnd.choice([1, 2, 5, 8, 13, 16]))
+    return m
+
+
+def random_config(rnd, big: bool) -> dict:
+    """A configuration drawn at random: one to five layers of any kind in any order, any span of them run one to three times, sizes of
+    the matrix-core kernels (``big``) or small odd ones, windows and blocks from one token up, with or without bigram table,
+    rotation, scaling and feed-forwards."""
+    layers = []
+    for _ in range(rnd.randint(1, 5)):
+        kind = rnd.choice(["attention", "delta", "parallel"])
+        if kind == "attention":
+            mixer = _random_attention(rnd, big, True)
+        elif kind == "delta":
+            kv_heads = rnd.choice([1, 2])
+            mixer = _delta(kv_heads * rnd.choice([1, 2]), kv_heads, rnd.choice([32, 64] if big else [5, 8, 17]), rnd.choice([32, 48] if big else [3, 9]),
+                           rnd.choice([1, 2, 3, 4]))
+        else:
+            heads = rnd.choice([1, 2, 5])
+            mixer = dict(left=_random_attention(rnd, big, False),
+                         right=_linear(heads, rnd.choice([32, 64] if big else [4, 9]), rnd.choice([16, 32] if big else [5, 6]),
+                                       [rnd.choice([1.0, 0.999, 0.9, 0.5]) for _ in range(heads)]))
+        layers.append(dict(type=kind, mixer=mixer, mlp=_dense(rnd.choice([16, 48, 72])) if rnd.random() < 0.8 else None))
+    conf = dict(architecture="Fotovik", vocab=rnd.choice([31, 90, 300]), width=rnd.choice([64, 128] if big else [24, 40, 56]),
+                norm=dict(eps=rnd.choice([1e-5, 1e-6, 3e-4])), embedding=dict(scale=rnd.choice([1.0, 3.0, 0.5])), layers=layers)
+    if rnd.random() < 0.8:
+        conf["embedding"]["bigram"] = dict(buckets=rnd.choice([7, 101, 1021]), mul_prev=rnd.choice([1, 127, 99991]), mul_cur=rnd.choice([1, 17, 77773]))
+    if rnd.random() < 0.7:
+        start = rnd.randint(0, len(layers) - 1)
+        conf["loop"] = dict(start=start, stop=rnd.randint(start + 1, len(layers)), times=rnd.randint(1, 3))
+    return conf
