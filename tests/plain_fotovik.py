@@ -82,17 +82,18 @@ def attention_head(q, k, v, scale, mask=None, sink=None):
     return out
 
 
-def attention(m, w, prefix, h, eps, layout, cached=lambda x: x):
-    """Grouped-query attention.  ``cached``: the rounding of what a cache would hold (keys after norm and rotation, values)."""
+def attention(m, w, prefix, h, eps, layout, cached=lambda x: x, stored=lambda x: x):
+    """Grouped-query attention.  ``cached``: the rounding of what a cache would hold (keys after norm and rotation, values); ``stored``: of
+    what separate kernels hand to each other (the projections, the rotated queries, the heads' outputs)."""
     T = h.shape[0]
     H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = (h @ w[prefix + "q"].to(F64).T).view(T, H, D)
-    k = (h @ w[prefix + "k"].to(F64).T).view(T, G, D)
-    v = (h @ w[prefix + "v"].to(F64).T).view(T, G, V)
+    q = stored(h @ w[prefix + "q"].to(F64).T).view(T, H, D)
+    k = stored(h @ w[prefix + "k"].to(F64).T).view(T, G, D)
+    v = stored(h @ w[prefix + "v"].to(F64).T).view(T, G, V)
     if prefix + "q.norm" in w:
         q = rms(q, eps) * w[prefix + "q.norm"].to(F64)
         k = rms(k, eps) * w[prefix + "k.norm"].to(F64)
-    q, k = rotate(q, m.get("rot"), layout), rotate(k, m.get("rot"), layout)
+    q, k = stored(rotate(q, m.get("rot"), layout)), rotate(k, m.get("rot"), layout)
     k, v = cached(k), cached(v)
     mask = (int(m["mask"]["size"]), int(m["mask"].get("pool", 0))) if m.get("mask") else None
     outs = []
@@ -100,7 +101,7 @@ def attention(m, w, prefix, h, eps, layout, cached=lambda x: x):
         g = i // (H // G)
         sink = w[prefix + "sink"].to(F64)[i] if prefix + "sink" in w else None
         outs.append(attention_head(q[:, i], k[:, g], v[:, g], float(m["scale"]), mask, sink))
-    return torch.cat(outs, -1) @ w[prefix + "o"].to(F64).T
+    return stored(torch.cat(outs, -1)) @ w[prefix + "o"].to(F64).T
 
 
 def short_conv(x, taps):
@@ -126,22 +127,22 @@ def delta_rule(q, k, v, beta, g):
     return out
 
 
-def delta_mixer(m, w, prefix, h, eps):
+def delta_mixer(m, w, prefix, h, eps, stored=lambda x: x):
     T = h.shape[0]
     H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    proj = {n: silu(short_conv(h @ w[prefix + n].to(F64).T, w[prefix + n + ".conv"].to(F64))) for n in "qkv"}
+    proj = {n: silu(short_conv(stored(h @ w[prefix + n].to(F64).T), w[prefix + n + ".conv"].to(F64))) for n in "qkv"}
     q, k, v = proj["q"].view(T, G, D), proj["k"].view(T, G, D), proj["v"].view(T, H, V)
     q = q / torch.sqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
     k = k / torch.sqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
     beta = torch.sigmoid(h @ w[prefix + "b"].to(F64).T)
     g = torch.exp(-torch.exp(w[prefix + "A_log"].to(F64)) * torch.nn.functional.softplus(h @ w[prefix + "a"].to(F64).T + w[prefix + "dt_bias"].to(F64)))
-    gate = silu(h @ w[prefix + "g"].to(F64).T).view(T, H, V)
+    gate = silu(stored(h @ w[prefix + "g"].to(F64).T)).view(T, H, V)
     outs = []
     for i in range(H):
         j = i // (H // G)
         o = delta_rule(q[:, j], k[:, j], v[:, i], beta[:, i], g[:, i])
         outs.append(rms(o, eps) * w[prefix + "norm"].to(F64) * gate[:, i])
-    return torch.cat(outs, -1) @ w[prefix + "o"].to(F64).T
+    return stored(torch.cat(outs, -1)) @ w[prefix + "o"].to(F64).T
 
 
 def lightning(q, k, v, decay):
@@ -154,35 +155,35 @@ def lightning(q, k, v, decay):
     return out
 
 
-def lightning_mixer(m, w, prefix, h, eps):
+def lightning_mixer(m, w, prefix, h, eps, stored=lambda x: x):
     T, H, D, V = h.shape[0], m["heads"], m["dim"], m["vdim"]
-    q = silu(h @ w[prefix + "q"].to(F64).T).view(T, H, D)
-    k = silu(h @ w[prefix + "k"].to(F64).T).view(T, H, D)
-    v = silu(h @ w[prefix + "v"].to(F64).T).view(T, H, V)
+    q = silu(stored(h @ w[prefix + "q"].to(F64).T)).view(T, H, D)
+    k = silu(stored(h @ w[prefix + "k"].to(F64).T)).view(T, H, D)
+    v = silu(stored(h @ w[prefix + "v"].to(F64).T)).view(T, H, V)
     o = torch.cat([lightning(q[:, i], k[:, i], v[:, i], float(m["decay"][i])) for i in range(H)], -1)
-    o = rms(o, eps) * w[prefix + "norm"].to(F64) * torch.sigmoid(h @ w[prefix + "g"].to(F64).T)
-    return o @ w[prefix + "o"].to(F64).T
+    o = rms(o, eps) * w[prefix + "norm"].to(F64) * torch.sigmoid(stored(h @ w[prefix + "g"].to(F64).T))
+    return stored(o) @ w[prefix + "o"].to(F64).T
 
 
-def parallel_mixer(m, w, prefix, h, eps, cached=lambda x: x):
-    left = attention(m["left"], w, prefix + "left.", h, eps, "halves", cached)
-    right = lightning_mixer(m["right"], w, prefix + "right.", h, eps)
+def parallel_mixer(m, w, prefix, h, eps, cached=lambda x: x, stored=lambda x: x):
+    left = stored(attention(m["left"], w, prefix + "left.", h, eps, "halves", cached, stored))
+    right = stored(lightning_mixer(m["right"], w, prefix + "right.", h, eps, stored))
     return 0.5 * (rms(left, eps) * w[prefix + "left.out"].to(F64) + rms(right, eps) * w[prefix + "right.out"].to(F64))
 
 
-def dense_ff(w, prefix, h):
-    z = h @ w[prefix + "up"].to(F64).T
-    return (0.5 * z * (1.0 + torch.erf(z / math.sqrt(2.0)))) @ w[prefix + "down"].to(F64).T
+def dense_ff(w, prefix, h, stored=lambda x: x):
+    z = stored(h @ w[prefix + "up"].to(F64).T)
+    return stored(0.5 * z * (1.0 + torch.erf(z / math.sqrt(2.0)))) @ w[prefix + "down"].to(F64).T
 
 
-def mixer(layer, w, prefix, h, eps, cached=lambda x: x):
+def mixer(layer, w, prefix, h, eps, cached=lambda x: x, stored=lambda x: x):
     kind = layer["type"]
     if kind == "attention":
-        return attention(layer["mixer"], w, prefix, h, eps, "pairs", cached)
+        return attention(layer["mixer"], w, prefix, h, eps, "pairs", cached, stored)
     if kind == "delta":
-        return delta_mixer(layer["mixer"], w, prefix, h, eps)
+        return delta_mixer(layer["mixer"], w, prefix, h, eps, stored)
     if kind == "parallel":
-        return parallel_mixer(layer["mixer"], w, prefix, h, eps, cached)
+        return parallel_mixer(layer["mixer"], w, prefix, h, eps, cached, stored)
     raise ValueError(kind)
 
 
@@ -210,10 +211,10 @@ def forward(config, w, tokens, cached=lambda x: x, stored=lambda x: x):
         layer, name = config["layers"][i], f"l{i}."
         if again:
             x = x + x0
-        y = stored(mixer(layer, w, name + "mix.", stored(rms(x, eps) * w[name + "norm1"].to(F64)), eps, cached))
+        y = stored(mixer(layer, w, name + "mix.", stored(rms(x, eps) * w[name + "norm1"].to(F64)), eps, cached, stored))
         x = x + rms(y, eps) * w[name + "norm1b"].to(F64)
         if layer.get("mlp"):
-            y = stored(dense_ff(w, name + "mlp.", stored(rms(x, eps) * w[name + "norm2"].to(F64))))
+            y = stored(dense_ff(w, name + "mlp.", stored(rms(x, eps) * w[name + "norm2"].to(F64)), stored))
             x = x + rms(y, eps) * w[name + "norm2b"].to(F64)
         after.append(x.clone())
     logits = stored(rms(x, eps) * w["final.norm"].to(F64)) @ w["head"].to(F64).T
