@@ -13,7 +13,8 @@ What it owns
 * **Block tables.**  Per request and group, the list of pages in logical order.  A group
   with a window gives pages back as soon as every key in them lies behind the window of
   all future queries (one with chunks: before the chunk of the next position); their table entries
-  fall back to the sentinel.
+  fall back to the sentinel.  A need that keeps a sequence's first positions beside its window
+  (``keep_first``) never gives back the pages that hold those.
 * **Slots.**  A request holds one slot from admission to release.  Runs that declare a
   :class:`~torchlet_amd.parts.base.StateNeed` get a tensor ``[slots + 1, *shape]``; a slot's
   rows are zeroed when it is handed out.  The last row (``pad_slot``) belongs to no request: the
@@ -223,7 +224,8 @@ class CacheManager:
         one the step writes.  ``None``: no bound (no window, or steps of any size)."""
         if not need.bounded or self.max_step_tokens is None:
             return None
-        return (need.reach + self.max_step_tokens - 2) // (self.page_size * need.stride) + 2
+        span = self.page_size * need.stride
+        return (need.reach + self.max_step_tokens - 2) // span + 2 + -(-need.keep_first // span)
 
     def _pool_size(self, need: PagedNeed) -> int:
         pages = self.num_pages
@@ -284,6 +286,11 @@ class CacheManager:
         if g.need.chunk is not None:          # the chunk that position `length` lies in starts here; later ones start later
             first = max(first, length // g.need.chunk * g.need.chunk)
         return first // g.span
+
+    @staticmethod
+    def _kept_blocks(g: _Group) -> int:
+        """Blocks at the start of a sequence that stay with the request whatever its length (they hold its kept first positions)."""
+        return -(-g.need.keep_first // g.span) if g.need.keep_first > 0 else 0
 
     def pages_missing(self, req_id, new_length: int) -> list[int]:
         """Per group, the pages that ``reserve(req_id, new_length)`` would take.  (A request's
@@ -354,7 +361,7 @@ class CacheManager:
             table = g.tables[req_id]
             first = min(self._first_live_block(g, new_length), len(table))
             was_first = min(self._first_live_block(g, old_length), first)     # blocks below were given back earlier
-            dead = [b for b in range(was_first, first) if table[b]]
+            dead = [b for b in range(max(was_first, self._kept_blocks(g)), first) if table[b]]
             g.pool.give([table[b] for b in dead])
             for b in dead:
                 table[b] = 0
@@ -405,9 +412,10 @@ class CacheManager:
         for gi, g in enumerate(self.groups):
             held: dict[int, object] = {}
             for req, table in g.tables.items():
-                pages = list(table)
+                kept = min(self._kept_blocks(g), len(table))
+                pages = list(table)[kept:]              # (the blocks of the kept first positions are held apart from the window's)
                 held_from = next((b for b, p in enumerate(pages) if p), len(pages))
-                if not all(pages[held_from:]):
+                if not all(pages[held_from:]) or not all(list(table)[:kept]):
                     raise CacheError(f"group {gi}: request {req!r} has a gap among its held pages")
                 for p in table:
                     if p == 0:

@@ -58,6 +58,20 @@ class ScalarRMSNormSpec(PartSpec):
 
 
 @dataclass(frozen=True)
+class OffsetRMSNormSpec(PartSpec):
+    """``x / sqrt(mean(x^2) + eps) * (offset + w) * gain`` with a weight vector ``w`` that is stored around zero (``offset`` 1) or as it
+    multiplies (``offset`` 0); ``gain``: one more fixed factor (a branch's share of the residual sum, where the norm follows a sublayer).
+    The norm folds a normed branch output and a second addend into the stream, so it may stand in blocks that norm their sublayers'
+    outputs.  ``weight_name`` as in :class:`RMSNormSpec`."""
+    kind: ClassVar[str] = "offset_rmsnorm"
+    dim: int = 0
+    eps: float = 1e-6
+    offset: float = 1.0
+    gain: float = 1.0
+    weight_name: str = "weight"
+
+
+@dataclass(frozen=True)
 class RotarySpec(PartSpec):
     """Split-half rotary position encoding over the whole head."""
     kind: ClassVar[str] = "rope_split_half"
@@ -82,9 +96,14 @@ class AttentionSpec(PartSpec):
 
 @dataclass(frozen=True)
 class SwiGLUSpec(PartSpec):
+    """``down(act(gate(h)) * up(h))`` without biases; ``activation``: ``silu`` or ``relu``; the three matrices' names below the part's."""
     kind: ClassVar[str] = "swiglu"
     hidden: int = 0
     intermediate: int = 0
+    activation: str = "silu"
+    gate_name: str = "gate_proj.weight"
+    up_name: str = "up_proj.weight"
+    down_name: str = "down_proj.weight"
 
 
 @dataclass(frozen=True)
@@ -105,6 +124,10 @@ class HalfRotarySpec(PartSpec):
     dims: int = 0
     base: float = 10000.0
     factor: float = 1.0
+    # ``bands = (factor, low, high, original)``: frequencies are scaled by their wavelength ``2 pi / f`` instead of all alike: shorter
+    # than ``original / high`` a frequency stays, longer than ``original / low`` it is divided by ``factor``, and between the two it is
+    # ``(1 - s) f / factor + s f`` with ``s = (original / wavelength - low) / (high - low)``
+    bands: tuple | None = None
 
 
 @dataclass(frozen=True)
@@ -141,6 +164,10 @@ class LatentAttentionSpec(PartSpec):
     norm_eps: float = 1e-6
     sink: bool = True
     position: PartSpec | None = None     # encoding of the rotated parts
+    # ``q_rank`` 0: no query latent, ``q = W_q h`` (tensor ``q``).  ``rot_dim`` 0: no rotated part.  ``window``: a query reads the last
+    # ``window`` positions, itself included.  ``gate``: head ``n``'s output is multiplied by ``sigmoid(W_g h)[n]`` (tensor ``g [heads, hidden]``).
+    window: int | None = None
+    gate: bool = False
 
 
 @dataclass(frozen=True)
@@ -170,6 +197,13 @@ class CappedAttentionSpec(PartSpec):
     qk_norm_eps: float = 1e-6
     sink: bool = False
     pool: int | None = None
+    # ``keep_first``: beside a window, a query also reads the first ``keep_first`` positions of its sequence (at their own positions).
+    # ``values_are_keys``: there is no value projection; the values are the keys as projected (bias added), before norm and rotation.
+    # ``qk_bias`` / ``o_bias``: the query and key projections / the output projection have biases (``q.b``, ``k.b``, ``o.b``).
+    keep_first: int = 0
+    values_are_keys: bool = False
+    qk_bias: bool = False
+    o_bias: bool = False
 
 
 @dataclass(frozen=True)
@@ -206,6 +240,24 @@ class GatedDeltaSpec(PartSpec):
 
 
 @dataclass(frozen=True)
+class SelectiveStateSpec(PartSpec):
+    """A selective state-space recurrence (Mamba-2): one projection gives per token ``[z | x | B | C | dt]`` (``heads * vdim`` twice, ``groups *
+    state`` twice, ``heads``); x, B and C pass a causal convolution of ``conv`` taps per channel with a bias, and silu; ``dt <- softplus(dt +
+    dt_bias)``; head ``n`` (reading B and C of group ``n // (heads / groups)``) moves its state ``S [state, vdim]`` by ``S <- exp(-exp(A_log) dt) S
+    + dt B x^T`` and gives ``y = S^T C + D x``; the heads side by side times ``silu(z)`` are divided by their root mean square in ``norm_groups``
+    equal parts (``norm_eps``), multiplied by a weight vector, and projected."""
+    kind: ClassVar[str] = "selective_state"
+    hidden: int = 0
+    heads: int = 0
+    vdim: int = 0
+    state: int = 0
+    groups: int = 1
+    conv: int = 4
+    norm_groups: int = 1
+    norm_eps: float = 1e-6
+
+
+@dataclass(frozen=True)
 class ParallelMixerSpec(PartSpec):
     """Several mixers side by side on the same input: ``sum_i scale_i * mixer_i(h)``.  ``branches``: ``(name, specification, scale)``
     of each; ``name`` is the branch's sub-module name in the checkpoint."""
@@ -233,9 +285,11 @@ class RoutedExpertsSpec(PartSpec):
     """``experts`` small feed-forward layers without biases, ``down(act(up(h)))`` or, ``gated``, ``down(act(gate(h)) * up(h))``; a linear
     router (in 32-bit; ``router_bias``: with a bias) scores them, the ``top`` largest scores per token are chosen and weigh the chosen
     experts' outputs.  ``scores``: ``"chosen"``: the choice goes by the logits and the weights are the softmax over the chosen ones alone;
-    ``"all"``: the scores are the softmax over all logits and the weights are the chosen experts' scores as they are.  ``choice_bias``: a
+    ``"all"``: the scores are the softmax over all logits and the weights are the chosen experts' scores as they are; ``"sigmoid"``: the
+    scores are the logits' sigmoids and the weights the chosen scores divided by their sum (plus ``weight_eps``).  ``choice_bias``: a
     vector ``correction`` is added to the scores for the choice only.  ``identity``: the router has that many outputs beyond ``experts``;
-    an expert chosen among those returns its input."""
+    an expert chosen among those returns its input.  ``weight_scale``: a factor on the weights.  ``shared``: the specification of one more
+    feed-forward (tensors below ``shared``) that runs for every token and is added to the experts' weighted sum."""
     kind: ClassVar[str] = "routed_experts"
     hidden: int = 0
     intermediate: int = 0
@@ -247,6 +301,9 @@ class RoutedExpertsSpec(PartSpec):
     scores: str = "chosen"
     choice_bias: bool = False
     identity: int = 0
+    weight_scale: float = 1.0
+    weight_eps: float = 1e-20
+    shared: PartSpec | None = None
 
 
 @dataclass(frozen=True)
@@ -341,6 +398,8 @@ class ModelSpec:
     position_table_name: str = ""  # a learned table ``[max_positions, hidden]`` whose row of the position is added to the (scaled) embedding; empty: none
     streams: int = 0               # copies of the residual that the blocks keep (hyper-connections); 0: the one plain residual
     bigram: HashedBigramSpec | None = None   # a hashed bigram row added to every token's (scaled) embedding
+    embed_norm: PartSpec | None = None       # a norm that the embedding's output passes before it becomes the stream
+    embed_norm_name: str = "embed.norm"
 
     def layer_name(self, i: int) -> str:
         return self.layers_format.format(i) if self.layers_format else f"{self.layers_prefix}.{i}"

@@ -450,27 +450,27 @@ extern "C" int tl_rope_cache_write(void* qkv, int row_stride, int tokens, int q_
 }
 
 // ------------------------------------------------------------------ SwiGLU gate
-// out[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu(g) = g / (1 + exp(-g)).
+// out[t, i] = act(gu[t, i]) * gu[t, inter + i]; act 0: silu(g) = g / (1 + exp(-g)), act 1: relu.
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total, int act) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const size_t t = idx / inter;
     const int i = (int)(idx % inter);
     const float g = to_float(gu[t * 2 * inter + i]);
     const float u = to_float(gu[t * 2 * inter + inter + i]);
-    out[idx] = from_float<T>(g / (1.f + expf(-g)) * u);
+    out[idx] = from_float<T>((act == 1 ? fmaxf(g, 0.f) : g / (1.f + expf(-g))) * u);
 }
 
-extern "C" int tl_swiglu(const void* gu, void* out, int tokens, int inter, int act_dtype, hipStream_t stream) {
-    TL_REQUIRE(tokens >= 0 && inter > 0, "swiglu: bad sizes tokens=%d inter=%d", tokens, inter);
+extern "C" int tl_swiglu(const void* gu, void* out, int tokens, int inter, int act_dtype, int act, hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && inter > 0 && (act == 0 || act == 1), "swiglu: bad sizes tokens=%d inter=%d, or an unknown gate %d", tokens, inter, act);
     const size_t total = (size_t)tokens * inter;
     if (total == 0) return TL_OK;
     dim3 block(256), grid((unsigned)((total + 255) / 256));
     if (act_dtype == TL_DT_F32)
-        swiglu_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, inter, total);
+        swiglu_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, inter, total, act);
     else if (act_dtype == TL_DT_BF16)
-        swiglu_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, total);
+        swiglu_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, total, act);
     else TL_REQUIRE(false, "swiglu: unknown dtype %d", act_dtype);
     TL_CHECK_LAUNCH("swiglu");
     return TL_OK;
@@ -835,5 +835,42 @@ extern "C" int tl_normed_sum(const void* x, int branches, int rows, int hidden, 
     else if (dtype == TL_DT_BF16) normed_sum_kernel<bf16_t><<<rows, 256, 0, stream>>>((const bf16_t*)x, branches, stride, (const float*)w, eps, (bf16_t*)out, hidden);
     else TL_REQUIRE(false, "normed_sum: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("normed_sum");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ embedding rows, normed
+// out[t, :] = r * rsqrt(mean(r^2) + eps) * weight[:] with r = float(table[ids[t], :]) * scale: a token's row enters the 32-bit stream through a
+// root-mean-square norm (weight: `hidden` floats).  One block per token, the row kept in shared memory between the two passes.
+template <typename T>
+__global__ void embedding_norm_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int hidden, int vocab,
+                                      float scale, const float* __restrict__ weight, float eps) {
+    extern __shared__ float en_row[];
+    __shared__ float red[16];
+    const int t = blockIdx.x;
+    int id = ids[t];
+    if (id < 0 || id >= vocab) id = 0;
+    const T* src = table + (size_t)id * hidden;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float v = to_float(src[i]) * scale;
+        en_row[i] = v;
+        ss = fmaf(v, v, ss);
+    }
+    const float inv = rsqrtf(block_sum(ss, red) / (float)hidden + eps);
+    float* dst = out + (size_t)t * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = en_row[i] * inv * weight[i];
+}
+
+extern "C" int tl_embedding_norm(const void* ids, const void* table, int table_dtype, void* out, int tokens, int hidden, int vocab, float scale,
+                                 const void* weight, float eps, hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && hidden > 0 && hidden <= 12288 && vocab > 0 && weight, "embedding_norm: bad sizes tokens=%d hidden=%d vocab=%d", tokens, hidden, vocab);
+    if (tokens == 0) return TL_OK;
+    const size_t smem = sizeof(float) * hidden;
+    if (table_dtype == TL_DT_F32)
+        embedding_norm_kernel<float><<<tokens, 256, smem, stream>>>((const int*)ids, (const float*)table, (float*)out, hidden, vocab, scale, (const float*)weight, eps);
+    else if (table_dtype == TL_DT_BF16)
+        embedding_norm_kernel<bf16_t><<<tokens, 256, smem, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab, scale, (const float*)weight, eps);
+    else TL_REQUIRE(false, "embedding_norm: unknown dtype %d", table_dtype);
+    TL_CHECK_LAUNCH("embedding_norm");
     return TL_OK;
 }

@@ -237,8 +237,11 @@ extern "C" int tl_grouped_gemm(const void* a, int a_ld, int a_group, const void*
 //   mode 0: the choice goes by the logits; the weights are the softmax over the chosen logits alone.
 //   mode 1: the scores are the softmax over all logits; the choice goes by score + bias[e] (bias optional), the weights are the
 //           chosen experts' scores as they are.
+//   mode 2: the scores are the logits' sigmoids; the choice goes by score + bias[e] (bias optional), the weights are the chosen
+//           experts' scores divided by their sum plus weight_eps.
+// In every mode the weights are multiplied by weight_scale at the end.
 __global__ void route_topk_kernel(const float* __restrict__ logits, int experts, int top, int mode, const float* __restrict__ bias,
-                                  int* __restrict__ chosen, float* __restrict__ weights, int tokens) {
+                                  int* __restrict__ chosen, float* __restrict__ weights, int tokens, float weight_scale, float weight_eps) {
     const int t = blockIdx.x * (blockDim.x / TL_WAVE) + threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
     if (t >= tokens) return;
     const float* z = logits + (size_t)t * experts;
@@ -259,6 +262,7 @@ __global__ void route_topk_kernel(const float* __restrict__ logits, int experts,
         for (int e = lane, i = 0; e < experts; e += TL_WAVE, ++i) {
             float v = z[e], sc = 0.f;
             if (mode == 1) { sc = expf(v - zmax) / den; v = bias ? sc + bias[e] : sc; }
+            else if (mode == 2) { sc = 1.f / (1.f + expf(-v)); v = bias ? sc + bias[e] : sc; }
             if (!((taken >> i) & 1ull) && (v > best || (v == best && e < at))) { best = v; at = e; score = sc; }
         }
 #pragma unroll
@@ -270,11 +274,11 @@ __global__ void route_topk_kernel(const float* __restrict__ logits, int experts,
         }
         if (at % TL_WAVE == lane) taken |= 1ull << (at / TL_WAVE);
         if (j == 0) first = best;
-        const float p = mode == 1 ? score : expf(best - first);
+        const float p = mode != 0 ? score : expf(best - first);
         sum += p;
         if (lane == j) { chosen[(size_t)t * top + j] = at; mine = p; }
     }
-    if (lane < top) weights[(size_t)t * top + lane] = mode == 1 ? mine : mine / sum;
+    if (lane < top) weights[(size_t)t * top + lane] = (mode == 1 ? mine : mode == 2 ? mine / (sum + weight_eps) : mine / sum) * weight_scale;
 }
 
 // Sort of the (token, choice) pairs by expert, by one work-group: offsets[e] .. offsets[e + 1] - 1 are the slots of
@@ -300,12 +304,13 @@ route_sort_kernel(const int* __restrict__ chosen, int pairs, int top, int expert
 }
 
 extern "C" int tl_route(const void* logits, int tokens, int experts, int top, int mode, const void* bias, void* chosen, void* weights,
-                        void* offsets, void* slot_token, void* pair_slot, hipStream_t stream) {
-    TL_REQUIRE(mode == 0 || mode == 1, "route: unknown mode %d", mode);
+                        void* offsets, void* slot_token, void* pair_slot, float weight_scale, float weight_eps, hipStream_t stream) {
+    TL_REQUIRE(mode >= 0 && mode <= 2, "route: unknown mode %d", mode);
     TL_REQUIRE(tokens >= 0 && experts > 0 && top > 0 && top <= experts && top <= TL_WAVE && experts <= 64 * TL_WAVE, "route: bad sizes (experts %d, top %d)", experts, top);
     TL_REQUIRE((experts + 1) * sizeof(int) <= 64 * 1024, "route: too many experts (%d)", experts);
     if (tokens == 0) return TL_OK;
-    route_topk_kernel<<<(tokens + 3) / 4, 4 * TL_WAVE, 0, stream>>>((const float*)logits, experts, top, mode, (const float*)bias, (int*)chosen, (float*)weights, tokens);
+    route_topk_kernel<<<(tokens + 3) / 4, 4 * TL_WAVE, 0, stream>>>((const float*)logits, experts, top, mode, (const float*)bias, (int*)chosen, (float*)weights, tokens,
+                                                                    weight_scale, weight_eps);
     TL_CHECK_LAUNCH("route_topk");
     route_sort_kernel<<<1, 1024, (experts + 1) * sizeof(int), stream>>>((const int*)chosen, tokens * top, top, experts, (int*)offsets,
                                                                        (int*)slot_token, (int*)pair_slot);
@@ -315,10 +320,12 @@ extern "C" int tl_route(const void* logits, int tokens, int experts, int top, in
 
 // ------------------------------------------------------------------ weighted sum of the chosen experts' outputs
 // out[t, :] = sum_j weights[t, j] * y[pair_slot[t * top + j], :], summed in the order of the choices.  With `x`: a pair whose slot is
-// offsets[real] or later chose an expert without tensors (an identity expert), and x[t, :] stands in for its row of y.
+// offsets[real] or later chose an expert without tensors (an identity expert), and x[t, :] stands in for its row of y.  With `addend`
+// (a shared expert's output): out[t, :] += addend[t, :], added last, in float.
 template <typename T>
 __global__ void combine_kernel(const T* __restrict__ y, const int* __restrict__ pair_slot, const float* __restrict__ weights,
-                               T* __restrict__ out, const T* __restrict__ x, const int* __restrict__ offsets, int real, int top, int width) {
+                               T* __restrict__ out, const T* __restrict__ x, const int* __restrict__ offsets, int real, int top, int width,
+                               const T* __restrict__ addend) {
     const int t = blockIdx.x;
     const int own_from = x ? offsets[real] : 0x7fffffff;
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
@@ -328,20 +335,21 @@ __global__ void combine_kernel(const T* __restrict__ y, const int* __restrict__ 
             const float v = slot >= own_from ? to_float(x[(size_t)t * width + i]) : to_float(y[(size_t)slot * width + i]);
             a = fmaf(weights[(size_t)t * top + j], v, a);
         }
+        if (addend) a += to_float(addend[(size_t)t * width + i]);
         out[(size_t)t * width + i] = from_float<T>(a);
     }
 }
 
 extern "C" int tl_combine(const void* y, const void* pair_slot, const void* weights, void* out, const void* x, const void* offsets, int real,
-                          int tokens, int top, int width, int dtype, hipStream_t stream) {
+                          int tokens, int top, int width, const void* addend, int dtype, hipStream_t stream) {
     TL_REQUIRE(tokens >= 0 && top > 0 && width > 0 && real >= 0 && (!x || offsets), "combine: bad sizes");
     if (tokens == 0) return TL_OK;
     if (dtype == TL_DT_F32)
         combine_kernel<float><<<tokens, 256, 0, stream>>>((const float*)y, (const int*)pair_slot, (const float*)weights, (float*)out, (const float*)x,
-                                                          (const int*)offsets, real, top, width);
+                                                          (const int*)offsets, real, top, width, (const float*)addend);
     else if (dtype == TL_DT_BF16)
         combine_kernel<bf16_t><<<tokens, 256, 0, stream>>>((const bf16_t*)y, (const int*)pair_slot, (const float*)weights, (bf16_t*)out, (const bf16_t*)x,
-                                                           (const int*)offsets, real, top, width);
+                                                           (const int*)offsets, real, top, width, (const bf16_t*)addend);
     else TL_REQUIRE(false, "combine: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("combine");
     return TL_OK;

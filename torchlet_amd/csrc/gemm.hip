@@ -490,7 +490,9 @@ constexpr int skinny_depth() {
     return d < 2 ? 2 : (d > 8 ? 8 : d);
 }
 
-__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + expf(-g)) * u; }
+// The gate of a fused gate/up product: GATE 1: silu(g) * u, GATE 2: relu(g) * u (the value of SW in the kernels below; 0: no gate).
+template <int GATE>
+__device__ __forceinline__ float gate_mul(float g, float u) { return GATE == 2 ? fmaxf(g, 0.f) * u : g / (1.f + expf(-g)) * u; }
 
 // SW (gate/up product with the SwiGLU gate applied to the accumulators): w holds blocks of 64
 // rows, 32 gate rows followed by the 32 up rows of the same columns; a work-group's strip is up to 16
@@ -572,7 +574,7 @@ struct NormArgs {
     float eps;
 };
 
-template <int R, int MT, int KS, typename TOut, bool SW = false, bool XL = false, int D = 2, bool RP = false, bool NF = false>
+template <int R, int MT, int KS, typename TOut, int SW = 0, bool XL = false, int D = 2, bool RP = false, bool NF = false>
 __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                               const void* __restrict__ bias, int bias_f32,
                                                               TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
@@ -832,7 +834,7 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
                 if (m < M) {
 #pragma unroll
                     for (int v = 0; v < 4; ++v)
-                        if (col + v < n_end) out[(size_t)m * ldo + col + v] = from_float<TOut>(silu_mul(gs[v], us[v]));
+                        if (col + v < n_end) out[(size_t)m * ldo + col + v] = from_float<TOut>(gate_mul<SW>(gs[v], us[v]));
                 }
             }
         } else {
@@ -938,7 +940,7 @@ static StripPlan plan_strips(int total, int most, int cap, bool even) {
 }
 
 // rows_per_strip > 0: one strip of that many outputs per work-group, whatever else holds.
-template <int R, int MT, int KS, typename TOut, bool SW, int D>
+template <int R, int MT, int KS, typename TOut, int SW, int D>
 static void launch_skinny_d(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                             int ldx, int ldo, int out_cols, hipStream_t stream, int rows_per_strip = 0) {
     const int total = SW ? out_cols : N;
@@ -968,7 +970,7 @@ static void launch_skinny_d(const void* x, const void* w, const void* bias, int 
 // A wave with many K steps ahead of it (a long K: the down projection) keeps as many in flight as
 // its registers hold; with a few steps (K of a hidden size) two are as good and start sooner
 // (measured at 3584 x 18944, one row: 33 -> 28 us with eight in flight; at 4608 x 3584: 11 -> 12.6 us).
-template <int R, int MT, int KS, typename TOut, bool SW>
+template <int R, int MT, int KS, typename TOut, int SW>
 static void launch_skinny_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                             int ldx, int ldo, int out_cols, hipStream_t stream, int rows_per_strip = 0) {
     constexpr int deep = skinny_depth<R, MT, KS>();
@@ -1073,7 +1075,7 @@ static TileChoice pick_tile(int M, int N) {
     return TILE_128x128_K64;
 }
 
-template <int BM, int BN, int WGM, int WGN, typename TOut, bool SW = false, int TK = 32>
+template <int BM, int BN, int WGM, int WGN, typename TOut, int SW = 0, int TK = 32>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tile_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                              const void* __restrict__ bias, int bias_f32,
                                                              TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
@@ -1184,7 +1186,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tile_kernel(const bf
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-                    if (m < M) out[(size_t)m * ldo + col] = from_float<TOut>(silu_mul(acc[i][j][v], acc[i][j + 1][v]));
+                    if (m < M) out[(size_t)m * ldo + col] = from_float<TOut>(gate_mul<SW>(acc[i][j][v], acc[i][j + 1][v]));
                 }
             }
         }
@@ -1208,7 +1210,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tile_kernel(const bf
 
 // Shared memory of a tile kernel: two buffers of (BM + BN) rows of TK + 8 elements.
 
-template <int BM, int BN, int WGM, int WGN, typename TOut, bool SW, int TK>
+template <int BM, int BN, int WGM, int WGN, typename TOut, int SW, int TK>
 static int launch_mfma_tile_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                               int ldx, int ldo, int out_cols, hipStream_t stream) {
     constexpr size_t lds = 2 * (size_t)(BM + BN) * (TK + 8) * sizeof(bf16_t);
@@ -1257,7 +1259,7 @@ constexpr int dl_slab_rows(int bm, int bn, int waves, int tk) {
     return (bm + bn + per - 1) / per * per;
 }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, bool SW = false, int TK = 64>
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, int SW = 0, int TK = 64>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                       const void* __restrict__ bias, int bias_f32,
                                                                       TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
@@ -1462,7 +1464,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
     const int c0 = (SW ? n0 / 2 : n0) + wn * WNO;           // first output column and row of this wave
     const int r0 = m0 + wm * WM;
     auto value = [&](int i, int jo, int v) -> float {
-        if constexpr (SW) return silu_mul(acc[i][2 * jo][v], acc[i][2 * jo + 1][v]);
+        if constexpr (SW) return gate_mul<SW>(acc[i][2 * jo][v], acc[i][2 * jo + 1][v]);
         else return acc[i][jo][v];
     };
     auto bias_at = [&](int n) -> float { return (!SW && bias && n < cols) ? load_vec(bias, bias_f32, n) : 0.f; };
@@ -1634,7 +1636,7 @@ static DlSplit plan_dl_split(int M, int N, int K) {
 }
 
 // parts > 1 (float results only): K is split into `parts` ranges of k_per columns and out holds that many [M, ldo] slabs.
-template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, bool SW, int TK = 64>
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, int SW, int TK = 64>
 static int launch_dl_tile_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                             int ldx, int ldo, int out_cols, hipStream_t stream, int parts = 1, int k_per = 0) {
     constexpr size_t lds = (size_t)STAGES * dl_slab_rows(BM, BN, WGM * WGN, TK) * TK * sizeof(bf16_t);
@@ -1652,7 +1654,7 @@ static int launch_dl_tile_t(const void* x, const void* w, const void* bias, int 
     return TL_OK;
 }
 
-template <typename TOut, bool SW>
+template <typename TOut, int SW>
 static int launch_dl_tile(DlTile tile, const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                           int ldx, int ldo, int out_cols, hipStream_t stream, int parts = 1, int k_per = 0) {
     switch (tile) {
@@ -1939,8 +1941,8 @@ extern "C" int tl_gemm_swiglu_normed(const void* residual, void* residual_out, c
 // of the same columns), padded with zero rows to a multiple of 64.  The gate is applied to the
 // float accumulators, as the reference's fused kernel does
 // (/root/reference/src/torchlet/v10_triton_paged_gqa/kernel/ffn_swiglu.py:139-160).
-extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, int I, int K, int ldx, int ldo,
-                              hipStream_t stream) {
+template <int GATE>
+static int gemm_gated(const void* x, const void* w, void* out, int M, int I, int K, int ldx, int ldo, hipStream_t stream) {
     TL_REQUIRE(M >= 0 && I > 0 && K > 0 && ldx >= K && ldo >= I, "gemm_swiglu: bad sizes M=%d I=%d K=%d", M, I, K);
     TL_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0,
                "gemm_swiglu: needs K and the row stride of x to be multiples of 8 and 16-byte aligned operands");
@@ -1953,23 +1955,29 @@ extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, in
     // as its weights: 32B sizes, 16 rows, 20.2 against 18.9 ms a step)
     const bool x_fits = M == 1 || (size_t)16 * 1024 + (size_t)M * (K + 8) * 2 <= 156 * 1024;
     if ((M <= 16 && (x_fits || K % 64 != 0)) || (M <= 32 && K % 64 != 0)) {
-        if (M <= 16) launch_skinny_t<1, 1, 16, bf16_t, true>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
-        else launch_skinny_t<1, 2, 16, bf16_t, true>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
+        if (M <= 16) launch_skinny_t<1, 1, 16, bf16_t, GATE>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
+        else launch_skinny_t<1, 2, 16, bf16_t, GATE>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
     } else if (K % 64 == 0) {
-        const int rc = launch_dl_tile<bf16_t, true>(pick_dl_tile(M, N, K, true), xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
+        const int rc = launch_dl_tile<bf16_t, GATE>(pick_dl_tile(M, N, K, true), xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
         if (rc != TL_OK) return rc;
     } else {
         int rc;
         switch (pick_tile(M, N)) {
-        case TILE_256x256: rc = launch_mfma_tile_t<256, 256, 4, 2, bf16_t, true, 64>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream); break;
-        case TILE_128x128_K32: rc = launch_mfma_tile_t<128, 128, 2, 2, bf16_t, true, 32>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream); break;
-        case TILE_128x128_K64: rc = launch_mfma_tile_t<128, 128, 2, 2, bf16_t, true, 64>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream); break;
-        default: rc = launch_mfma_tile_t<64, 128, 2, 2, bf16_t, true, 64>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream); break;
+        case TILE_256x256: rc = launch_mfma_tile_t<256, 256, 4, 2, bf16_t, GATE, 64>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream); break;
+        case TILE_128x128_K32: rc = launch_mfma_tile_t<128, 128, 2, 2, bf16_t, GATE, 32>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream); break;
+        case TILE_128x128_K64: rc = launch_mfma_tile_t<128, 128, 2, 2, bf16_t, GATE, 64>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream); break;
+        default: rc = launch_mfma_tile_t<64, 128, 2, 2, bf16_t, GATE, 64>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream); break;
         }
         if (rc != TL_OK) return rc;
     }
     TL_CHECK_LAUNCH("gemm_swiglu");
     return TL_OK;
+}
+
+// `act`: the gate's activation, 0 silu, 1 relu.
+extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, int I, int K, int ldx, int ldo, int act, hipStream_t stream) {
+    TL_REQUIRE(act == 0 || act == 1, "gemm_swiglu: unknown gate %d", act);
+    return act == 1 ? gemm_gated<2>(x, w, out, M, I, K, ldx, ldo, stream) : gemm_gated<1>(x, w, out, M, I, K, ldx, ldo, stream);
 }
 
 // out[P, M, N] (float) = partial sums of x w^T over P ranges of K, for a product with too few output

@@ -20,11 +20,12 @@ __device__ __forceinline__ void turn_pair(float u, float v, float pos, float f, 
 }
 
 // ------------------------------------------------------------------ norms of the two latents, rotation, cache write
-// down [tokens, ld]: q_rank numbers of the query latent, then rank of the key/value latent, then rot of the shared key part.
-// cq = rmsnorm(first q_rank) * wq;  page row of the token = [rmsnorm(next rank) * wkv, the last rot with the first
+// down [tokens, ld]: q_rank numbers of the query latent (q_rank 0: none), and from column kv_off on rank numbers of the key/value
+// latent, then rot of the shared key part.
+// cq = rmsnorm(first q_rank) * wq;  page row of the token = [rmsnorm(the rank numbers) * wkv, the last rot with the first
 // rot_dims of them turned in pairs].  A token whose block-table entry is 0 (the sentinel page) writes nothing.
 template <typename T>
-__global__ void latent_prepare_kernel(const T* __restrict__ down, int ld, int q_rank, int rank, int rot, int rot_dims,
+__global__ void latent_prepare_kernel(const T* __restrict__ down, int ld, int q_rank, int kv_off, int rank, int rot, int rot_dims,
                                       const void* __restrict__ wq, int wq_f32, const void* __restrict__ wkv, int wkv_f32, float eps,
                                       const int* __restrict__ positions, const float* __restrict__ inv_freq,
                                       const int* __restrict__ token_req, const int* __restrict__ block_table, int bt_stride,
@@ -32,24 +33,26 @@ __global__ void latent_prepare_kernel(const T* __restrict__ down, int ld, int q_
     __shared__ float red[16];
     const int t = blockIdx.x;
     const T* row = down + (size_t)t * ld;
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < q_rank; i += blockDim.x) { const float x = to_float(row[i]); ss = fmaf(x, x, ss); }
-    ss = block_sum(ss, red);
-    float inv = 1.f / sqrtf(ss / (float)q_rank + eps);
-    for (int i = threadIdx.x; i < q_rank; i += blockDim.x)
-        cq[(size_t)t * q_rank + i] = from_float<T>(to_float(row[i]) * inv * load_vec(wq, wq_f32, i));
+    float ss = 0.f, inv = 0.f;
+    if (q_rank > 0) {
+        for (int i = threadIdx.x; i < q_rank; i += blockDim.x) { const float x = to_float(row[i]); ss = fmaf(x, x, ss); }
+        ss = block_sum(ss, red);
+        inv = 1.f / sqrtf(ss / (float)q_rank + eps);
+        for (int i = threadIdx.x; i < q_rank; i += blockDim.x)
+            cq[(size_t)t * q_rank + i] = from_float<T>(to_float(row[i]) * inv * load_vec(wq, wq_f32, i));
+    }
     if (plane == nullptr) return;
     const int pos = positions[t];
     const int page = block_table[(size_t)token_req[t] * bt_stride + pos / page_size];
     ss = 0.f;
-    for (int i = threadIdx.x; i < rank; i += blockDim.x) { const float x = to_float(row[q_rank + i]); ss = fmaf(x, x, ss); }
+    for (int i = threadIdx.x; i < rank; i += blockDim.x) { const float x = to_float(row[kv_off + i]); ss = fmaf(x, x, ss); }
     ss = block_sum(ss, red);
     if (page == 0) return;
     inv = 1.f / sqrtf(ss / (float)rank + eps);
     T* dst = plane + ((size_t)page * page_size + pos % page_size) * (rank + rot);
     for (int i = threadIdx.x; i < rank; i += blockDim.x)
-        dst[i] = from_float<T>(to_float(row[q_rank + i]) * inv * load_vec(wkv, wkv_f32, i));
-    const T* kr = row + q_rank + rank;
+        dst[i] = from_float<T>(to_float(row[kv_off + i]) * inv * load_vec(wkv, wkv_f32, i));
+    const T* kr = row + kv_off + rank;
     for (int i = threadIdx.x; i < rot_dims / 2; i += blockDim.x) {
         float a, b;
         turn_pair(to_float(kr[2 * i]), to_float(kr[2 * i + 1]), (float)pos, inv_freq[i], a, b);
@@ -59,16 +62,17 @@ __global__ void latent_prepare_kernel(const T* __restrict__ down, int ld, int q_
     for (int i = rot_dims + threadIdx.x; i < rot; i += blockDim.x) dst[rank + i] = kr[i];
 }
 
-extern "C" int tl_latent_prepare(const void* down, int ld, int q_rank, int rank, int rot, int rot_dims, const void* wq, int wq_f32,
+extern "C" int tl_latent_prepare(const void* down, int ld, int q_rank, int kv_off, int rank, int rot, int rot_dims, const void* wq, int wq_f32,
                                  const void* wkv, int wkv_f32, float eps, const void* positions, const void* inv_freq,
                                  const void* token_req, const void* block_table, int bt_stride, void* plane, int page_size,
                                  void* cq, int tokens, int dtype, hipStream_t stream) {
-    TL_REQUIRE(tokens >= 0 && q_rank > 0 && rank > 0 && rot >= 0 && rot_dims % 2 == 0 && rot_dims <= rot && ld >= q_rank + rank + rot,
+    TL_REQUIRE(tokens >= 0 && q_rank >= 0 && kv_off >= q_rank && rank > 0 && rot >= 0 && rot_dims % 2 == 0 && rot_dims <= rot && ld >= kv_off + rank + rot,
                "latent_prepare: bad sizes");
+    TL_REQUIRE(q_rank == 0 || (wq && cq), "latent_prepare: a query latent needs its norm's weight and a place to go");
     TL_REQUIRE(plane == nullptr || (page_size > 0 && block_table != nullptr && token_req != nullptr), "latent_prepare: a cache write needs the block table");
     if (tokens == 0) return TL_OK;
     dim3 grid(tokens), block(256);
-#define TL_ARGS(T) (const T*)down, ld, q_rank, rank, rot, rot_dims, wq, wq_f32, wkv, wkv_f32, eps, (const int*)positions, (const float*)inv_freq, \
+#define TL_ARGS(T) (const T*)down, ld, q_rank, kv_off, rank, rot, rot_dims, wq, wq_f32, wkv, wkv_f32, eps, (const int*)positions, (const float*)inv_freq, \
                    (const int*)token_req, (const int*)block_table, bt_stride, (T*)plane, page_size, (T*)cq
     if (dtype == TL_DT_F32) latent_prepare_kernel<float><<<grid, block, 0, stream>>>(TL_ARGS(float));
     else if (dtype == TL_DT_BF16) latent_prepare_kernel<bf16_t><<<grid, block, 0, stream>>>(TL_ARGS(bf16_t));
@@ -137,7 +141,7 @@ latent_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, 
                         const int* __restrict__ block_table, int bt_stride, const int* __restrict__ req_indptr,
                         const int* __restrict__ ctx_lens, const int* __restrict__ tile_req, const int* __restrict__ tile_tok0,
                         int tile_tokens, int heads, int rank, int rot, int page_size, float scale, const float* __restrict__ sink,
-                        int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+                        int splits, float* __restrict__ part_o, float* __restrict__ part_ml, int window, const T* __restrict__ gate, int gate_ld) {
     extern __shared__ float smem[];
     const int D = rank + rot, ldk = D + 1;             // a row more than a multiple of the banks apart: lanes read rows side by side
     float* sk = smem;                                  // [KT][ldk]
@@ -168,7 +172,11 @@ latent_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, 
     float m = with_sink ? sink[rh] : -INFINITY, l = with_sink ? 1.f : 0.f;
     const int last = ctx + tok0 + ntok - 1;            // the last key any row of the tile sees
     const int* table = block_table + (size_t)req * bt_stride;
-    for (int k0 = split * LAT_KT; k0 <= last; k0 += splits * LAT_KT) {
+    // with a window a row at qpos reads the keys qpos - window + 1 .. qpos; the tile starts at the step of LAT_KT keys (counted from
+    // position 0, so that a key's step does not depend on the tile) in which its first row's first key lies
+    const int kbegin = window > 0 ? max(0, ctx + tok0 - window + 1) / LAT_KT * LAT_KT : 0;
+    const int qfirst = window > 0 ? max(0, qpos - window + 1) : 0;
+    for (int k0 = kbegin + split * LAT_KT; k0 <= last; k0 += splits * LAT_KT) {
         __syncthreads();
         const int nk = min(LAT_KT, last + 1 - k0);
         for (int i = threadIdx.x; i < nk * D; i += blockDim.x) {
@@ -177,10 +185,10 @@ latent_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, 
             sk[kk * ldk + d] = to_float(plane[((size_t)page * page_size + pos % page_size) * D + d]);
         }
         __syncthreads();
-        if (!row_ok || k0 > qpos) continue;
+        if (!row_ok || k0 > qpos || k0 + nk <= qfirst) continue;
         // scores: lanes 0..KT-1 take one key each (the upper half of the wave idles here)
         float s = -INFINITY;
-        if (lane < nk && k0 + lane <= qpos) {
+        if (lane < nk && k0 + lane <= qpos && k0 + lane >= qfirst) {
             const float* kr = sk + lane * ldk;
             const float* qr = sq + wave * D;
             float dot = 0.f;
@@ -210,7 +218,8 @@ latent_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, 
     }
     if (!row_ok) return;
     if (splits == 1) {
-        const float inv = l > 0.f ? 1.f / l : 0.f;
+        float inv = l > 0.f ? 1.f / l : 0.f;
+        if (gate) inv *= 1.f / (1.f + expf(-to_float(gate[(size_t)tok * gate_ld + rh])));
         T* o = out + ((size_t)tok * heads + rh) * rank;
 #pragma unroll
         for (int c = 0; c < 16; ++c) {
@@ -235,7 +244,7 @@ latent_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, 
 #define LAT_MAX_SPLITS 64
 template <typename T>
 __global__ void latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, T* __restrict__ out,
-                                    int rows, int rank, int splits) {
+                                    int rows, int rank, int splits, const T* __restrict__ gate, int gate_ld, int heads) {
     __shared__ float wgt[LAT_MAX_SPLITS];
     __shared__ float inv_s;
     const int row = blockIdx.x;
@@ -251,7 +260,11 @@ __global__ void latent_merge_kernel(const float* __restrict__ part_o, const floa
             const float wi = __shfl(w, i, TL_WAVE), li = ml[i * 2 + 1];
             den += wi * li;
         }
-        if (s == 0) inv_s = den > 0.f ? 1.f / den : 0.f;
+        if (s == 0) {
+            float inv0 = den > 0.f ? 1.f / den : 0.f;
+            if (gate) inv0 *= 1.f / (1.f + expf(-to_float(gate[(size_t)(row / heads) * gate_ld + row % heads])));
+            inv_s = inv0;
+        }
     }
     __syncthreads();
     const float inv = inv_s;
@@ -291,7 +304,8 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
                              const int* __restrict__ block_table, int bt_stride, const int* __restrict__ req_indptr,
                              const int* __restrict__ ctx_lens, const int* __restrict__ tile_req, const int* __restrict__ tile_tok0,
                              int tile_tokens, int heads, int rank, int rot, int page_size, float scale, const float* __restrict__ sink,
-                             int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+                             int splits, float* __restrict__ part_o, float* __restrict__ part_ml, int window, const bf16_t* __restrict__ gate,
+                             int gate_ld) {
     constexpr int WPR = 4 / RB;                      // waves that share a block of rows
     constexpr int NT = 32 / WPR;                     // most blocks of 16 latent columns a wave sums (latents of up to 512 numbers)
     extern __shared__ __align__(16) unsigned char lm_smem[];
@@ -312,6 +326,7 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
     const bool row_ok = row < rows;
     const int rt = row_ok ? row / hchunk : 0, rh = head0 + (row_ok ? row % hchunk : 0);
     const int tok = first + tok0 + rt, qpos = ctx + tok0 + rt;
+    const int qfirst = window > 0 ? max(0, qpos - window + 1) : 0;      // the first key this query reads
     LmFrag qf[LM_DC_MAX];
 #pragma unroll
     for (int c = 0; c < LM_DC_MAX; ++c)
@@ -418,8 +433,8 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const int key = kbase + 4 * g + v;
-                    sc[v] = (row_ok && key <= qpos) ? s00[v] * scale2 : -INFINITY;
-                    sc[4 + v] = (row_ok && key + 16 <= qpos) ? s10[v] * scale2 : -INFINITY;
+                    sc[v] = (row_ok && key <= qpos && key >= qfirst) ? s00[v] * scale2 : -INFINITY;
+                    sc[4 + v] = (row_ok && key + 16 <= qpos && key + 16 >= qfirst) ? s10[v] * scale2 : -INFINITY;
                 }
             }
             float mloc = sc[0];
@@ -428,7 +443,7 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
             mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
             const float m_new = fmaxf(m, mloc);
-            const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+            const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);     // (m_new may still be -inf: a step wholly before this query's window)
             const bool moved = __any(m_new != m);    // the sums are rescaled only when some query's maximum moved
             LmFrag pf;
             float psum = 0.f;
@@ -454,7 +469,8 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
             }
         }
     };
-    const int kfirst = split * LM_KEYS;
+    // (with a window the tile starts at the step, counted from position 0, in which its first token's first key lies)
+    const int kfirst = (window > 0 ? max(0, ctx + tok0 - window + 1) / LM_KEYS * LM_KEYS : 0) + split * LM_KEYS;
     if (kfirst <= last) request(stage0, kfirst);
     if constexpr (TWO) {
         if (kfirst + stride <= last) request(stage1, kfirst + stride);
@@ -469,7 +485,8 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
     l += __shfl_xor(l, 32, 64);
     if (!row_ok) return;
     if (splits == 1) {
-        const float inv = l > 0.f ? 1.f / l : 0.f;
+        float inv = l > 0.f ? 1.f / l : 0.f;
+        if (gate) inv *= 1.f / (1.f + expf(-to_float(gate[(size_t)tok * gate_ld + rh])));
         bf16_t* o = out + ((size_t)tok * heads + rh) * rank;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
@@ -503,7 +520,8 @@ static bool lm_fits(int rank, int rot, int q_ld, const void* q, const void* plan
 template <int RB>
 static int launch_lm(const void* q, int q_ld, void* out, const void* plane, const void* block_table, int bt_stride, const void* req_indptr,
                      const void* ctx_lens, const void* tile_req, const void* tile_tok0, int num_tiles, int tile_tokens, int heads, int rank,
-                     int rot, int page_size, float scale, const void* sink, int splits, void* part_o, void* part_ml, hipStream_t stream) {
+                     int rot, int page_size, float scale, const void* sink, int splits, void* part_o, void* part_ml, int window, const void* gate,
+                     int gate_ld, hipStream_t stream) {
     static size_t allowed = 48 * 1024;               // (per instance of the template)
     const size_t smem = lm_smem_bytes(rank, rot);
     auto kernel = latent_attention_mfma_kernel<RB>;
@@ -516,7 +534,8 @@ static int launch_lm(const void* q, int q_ld, void* out, const void* plane, cons
     dim3 grid(num_tiles, (heads + 15) / 16, splits), block(256);
     kernel<<<grid, block, smem, stream>>>((const bf16_t*)q, q_ld, (bf16_t*)out, (const bf16_t*)plane, (const int*)block_table, bt_stride,
                                           (const int*)req_indptr, (const int*)ctx_lens, (const int*)tile_req, (const int*)tile_tok0, tile_tokens,
-                                          heads, rank, rot, page_size, scale, (const float*)sink, splits, (float*)part_o, (float*)part_ml);
+                                          heads, rank, rot, page_size, scale, (const float*)sink, splits, (float*)part_o, (float*)part_ml, window,
+                                          (const bf16_t*)gate, gate_ld);
     TL_CHECK_LAUNCH("latent_attention_mfma");
     return TL_OK;
 }
@@ -528,11 +547,14 @@ extern "C" int tl_latent_attention_mfma_fits(int rank, int rot, int q_ld) {
 
 // q [tokens, q_ld]: per head rank + rot numbers (head h at column h * (rank + rot)); out [tokens, heads * rank];
 // plane [pages, page_size, rank + rot]; sink float [heads] or null; tile_req null: tile i is the one token of request i.
+// window > 0: a query reads its last `window` keys only, itself included.  gate (of the activation type, [tokens, gate_ld], or null):
+// head h's output of token t is multiplied by sigmoid(gate[t, h]).
 extern "C" int tl_latent_attention(const void* q, int q_ld, void* out, const void* plane, const void* block_table, int bt_stride,
                                    const void* req_indptr, const void* ctx_lens, const void* tile_req, const void* tile_tok0,
                                    int num_tiles, int tokens, int tile_tokens, int heads, int rank, int rot, int page_size, float scale,
                                    const void* sink, int splits, void* part_o, void* part_ml, int dtype, int general, int max_new_tokens,
-                                   hipStream_t stream) {
+                                   int window, const void* gate, int gate_ld, hipStream_t stream) {
+    TL_REQUIRE(window >= 0 && (!gate || gate_ld >= heads), "latent_attention: a window is not negative and a gate has a number per head");
     TL_REQUIRE(num_tiles >= 0 && heads > 0 && rank > 0 && rot >= 0 && page_size > 0 && tile_tokens > 0, "latent_attention: bad sizes");
     TL_REQUIRE(rank <= 16 * TL_WAVE, "latent_attention: built for latents of up to %d numbers, got %d", 16 * TL_WAVE, rank);
     TL_REQUIRE(splits >= 1 && splits <= LAT_MAX_SPLITS && (splits == 1 || (part_o != nullptr && part_ml != nullptr)), "latent_attention: 1 to 64 parts, with their scratch");
@@ -543,13 +565,14 @@ extern "C" int tl_latent_attention(const void* q, int q_ld, void* out, const voi
         TL_REQUIRE(tile_tokens * min(heads, 16) <= 64, "latent_attention: a tile of %d tokens and %d heads has more than 64 rows", tile_tokens, heads);
         int rc;
 #define TL_LM(RB) rc = launch_lm<RB>(q, q_ld, out, plane, block_table, bt_stride, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles, tile_tokens, \
-                                     heads, rank, rot, page_size, scale, sink, splits, part_o, part_ml, stream)
+                                     heads, rank, rot, page_size, scale, sink, splits, part_o, part_ml, window, gate, gate_ld, stream)
         if (tile_rows <= 16) TL_LM(1); else if (tile_rows <= 32) TL_LM(2); else TL_LM(4);
 #undef TL_LM
         if (rc != TL_OK) return rc;
         if (splits > 1) {
             const int rows = tokens * heads;
-            latent_merge_kernel<bf16_t><<<rows, 128, 0, stream>>>((const float*)part_o, (const float*)part_ml, (bf16_t*)out, rows, rank, splits);
+            latent_merge_kernel<bf16_t><<<rows, 128, 0, stream>>>((const float*)part_o, (const float*)part_ml, (bf16_t*)out, rows, rank, splits,
+                                                                  (const bf16_t*)gate, gate_ld, heads);
             TL_CHECK_LAUNCH("latent_merge");
         }
         return TL_OK;
@@ -561,7 +584,7 @@ extern "C" int tl_latent_attention(const void* q, int q_ld, void* out, const voi
     dim3 grid(num_tiles, (heads + LAT_ROWS - 1) / LAT_ROWS, splits), block(LAT_ROWS * TL_WAVE);
 #define TL_ARGS(T) (const T*)q, q_ld, (T*)out, (const T*)plane, (const int*)block_table, bt_stride, (const int*)req_indptr, (const int*)ctx_lens, \
                    (const int*)tile_req, (const int*)tile_tok0, tile_tokens, heads, rank, rot, page_size, scale, (const float*)sink, splits,      \
-                   (float*)part_o, (float*)part_ml
+                   (float*)part_o, (float*)part_ml, window, (const T*)gate, gate_ld
     if (dtype == TL_DT_F32) {
         auto kernel = latent_attention_kernel<float>;
         if (smem > 48 * 1024 && hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
@@ -579,8 +602,10 @@ extern "C" int tl_latent_attention(const void* q, int q_ld, void* out, const voi
     TL_CHECK_LAUNCH("latent_attention");
     if (splits > 1) {
         const int rows = tokens * heads;
-        if (dtype == TL_DT_F32) latent_merge_kernel<float><<<rows, 128, 0, stream>>>((const float*)part_o, (const float*)part_ml, (float*)out, rows, rank, splits);
-        else latent_merge_kernel<bf16_t><<<rows, 128, 0, stream>>>((const float*)part_o, (const float*)part_ml, (bf16_t*)out, rows, rank, splits);
+        if (dtype == TL_DT_F32) latent_merge_kernel<float><<<rows, 128, 0, stream>>>((const float*)part_o, (const float*)part_ml, (float*)out, rows, rank, splits,
+                                                                                     (const float*)gate, gate_ld, heads);
+        else latent_merge_kernel<bf16_t><<<rows, 128, 0, stream>>>((const float*)part_o, (const float*)part_ml, (bf16_t*)out, rows, rank, splits,
+                                                                   (const bf16_t*)gate, gate_ld, heads);
         TL_CHECK_LAUNCH("latent_merge");
     }
     return TL_OK;

@@ -53,6 +53,7 @@ extern "C" int tl_kv_cache_write(const void* k, int k_ld, const void* v, int v_l
 // ------------------------------------------------------------------ the mask and the cap
 struct LocalMask {
     int chunk, window;
+    int keep_first;          // beside a window: the positions 0 .. keep_first - 1 are read by every later query, at their own places
     // the first key a query at position p reads
     __device__ __forceinline__ int first(int p) const {
         int lo = 0;
@@ -99,15 +100,16 @@ local_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, i
     float acc[LA_COLS];
 #pragma unroll
     for (int c = 0; c < LA_COLS; ++c) acc[c] = 0.f;
-    const int nkeys = npool + p - lo + 1;
+    const int nkept = min(mask.keep_first, lo);          // kept first tokens that lie before the window: keys npool .. npool + nkept - 1
+    const int nkeys = npool + nkept + p - lo + 1;
     for (int b = wave; b * TL_WAVE < nkeys; b += LA_WAVES) {
-        const int u = b * TL_WAVE + lane;                // pooled blocks first, then the tokens lo .. p
+        const int u = b * TL_WAVE + lane;                // pooled blocks first, then the kept first tokens, then the tokens lo .. p
         const bool ok = u < nkeys;
         float s = -INFINITY;
         const T* vr0 = v_plane;                          // the key's values: column c at vr0[c * page_size]
         if (ok) {
             const bool pooled = u < npool;
-            const int j = pooled ? u : lo + u - npool;
+            const int j = pooled ? u : (u < npool + nkept ? u - npool : lo + u - npool - nkept);
             const int page = (pooled ? ptable : table)[j / page_size];
             const size_t at = (size_t)page * kv_heads + g;
             const int slot = j % page_size;
@@ -333,6 +335,11 @@ local_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __re
         if (n_tile_blocks > 0)
             run(pk_plane, pv_plane, pool_table + (size_t)req * pool_table_ld, pool_table_width, 0, n_tile_blocks - 1, 0, n_my_blocks - 1);
     }
+    if (mask.keep_first > 0 && mask.window > 0) {
+        // the kept first tokens that lie before a token's window: 0 .. min(keep_first, its window's start) - 1; the tile's last token reads the most
+        const int n_tile_kept = min(mask.keep_first, mask.first(p_last)), n_my_kept = min(mask.keep_first, my_lo);
+        if (n_tile_kept > 0) run(k_plane, v_plane, table, table_width, 0, n_tile_kept - 1, 0, n_my_kept - 1);
+    }
     // the first token reads furthest back; pages before may be gone
     run(k_plane, v_plane, table, table_width, mask.first(p0), p_last, my_lo, my_p);
     l += __shfl_xor(l, 16, TL_WAVE);
@@ -399,7 +406,8 @@ extern "C" int tl_local_attention_tiles(const void* q, int q_ld, void* out, int 
                                         const void* tile_req, const void* tile_tok0, int tiles, int heads, int kv_heads, int dim, int vdim,
                                         int page_size, float scale, float cap, int chunk, int window, float gain, const void* sink,
                                         const void* pk_plane, const void* pv_plane, const void* pool_table, int pool_table_ld, int pool_table_width,
-                                        int pool, hipStream_t stream) {
+                                        int pool, int keep_first, hipStream_t stream) {
+    TL_REQUIRE(keep_first >= 0 && (keep_first == 0 || (window > 0 && chunk == 0)), "local_attention_tiles: kept first tokens stand beside a window, without chunks");
     TL_REQUIRE(pool >= 0 && (pool == 0 || (window > 0 && pk_plane && pv_plane && pool_table && pool_table_ld >= pool_table_width && pool_table_width > 0)),
                "local_attention_tiles: pooled blocks need a window, their planes and their block table");
     TL_REQUIRE(tiles >= 0 && heads > 0 && heads <= 65535 && kv_heads > 0 && heads % kv_heads == 0 && page_size > 0, "local_attention_tiles: bad sizes");
@@ -407,7 +415,7 @@ extern "C" int tl_local_attention_tiles(const void* q, int q_ld, void* out, int 
     TL_REQUIRE(q_ld >= heads * dim && q_ld % 8 == 0 && ((uintptr_t)q & 15) == 0 && out_ld >= heads * vdim && table_ld >= table_width && chunk >= 0 && window >= 0,
                "local_attention_tiles: rows too short or not aligned");
     if (tiles == 0) return TL_OK;
-    const LocalMask mask{chunk, window};
+    const LocalMask mask{chunk, window, keep_first};
 #define TL_LAM(DK, DV)                                                                                                                      \
     launch_local_mfma<DK, DV>(q, q_ld, out, out_ld, k_plane, v_plane, block_table, table_ld, table_width, req_indptr, ctx_lens, tile_req,  \
                               tile_tok0, tiles, heads, kv_heads, page_size, scale, cap, mask, gain, sink, pk_plane, pv_plane, pool_table,        \
@@ -440,14 +448,15 @@ extern "C" int tl_local_attention(const void* q, int q_ld, void* out, int out_ld
                                   const void* block_table, int table_ld, int table_width, const void* token_req, const void* positions,
                                   int tokens, int heads, int kv_heads, int dim, int vdim, int page_size, float scale, float cap, int chunk,
                                   int window, float gain, const void* sink, const void* pk_plane, const void* pv_plane, const void* pool_table,
-                                  int pool_table_ld, int pool, int dtype, hipStream_t stream) {
+                                  int pool_table_ld, int pool, int keep_first, int dtype, hipStream_t stream) {
+    TL_REQUIRE(keep_first >= 0 && (keep_first == 0 || (window > 0 && chunk == 0)), "local_attention: kept first tokens stand beside a window, without chunks");
     TL_REQUIRE(pool >= 0 && (pool == 0 || (window > 0 && pk_plane && pv_plane && pool_table)), "local_attention: pooled blocks need a window, their planes and their block table");
     TL_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0 && page_size > 0, "local_attention: bad sizes");
     TL_REQUIRE(dim <= LA_MAX_DIM && vdim <= LA_MAX_DIM, "local_attention: built for heads of up to %d numbers, got %d / %d", LA_MAX_DIM, dim, vdim);
     TL_REQUIRE(q_ld >= heads * dim && out_ld >= heads * vdim && table_ld >= table_width && chunk >= 0 && window >= 0, "local_attention: rows too short");
     TL_REQUIRE(heads <= 65535, "local_attention: too many heads");
     if (tokens == 0) return TL_OK;
-    const LocalMask mask{chunk, window};
+    const LocalMask mask{chunk, window, keep_first};
     dim3 grid(tokens, heads), block(LA_WAVES * TL_WAVE);
     if (dtype == TL_DT_F32)
         local_attention_kernel<float><<<grid, block, 0, stream>>>((const float*)q, q_ld, (float*)out, out_ld, (const float*)k_plane, (const float*)v_plane,
@@ -532,12 +541,14 @@ extern "C" int tl_pool_blocks(const void* k_plane, const void* v_plane, int page
 //   norm (norm_a / norm_b != null): v <- v / sqrt(mean(v^2) + eps) * w[d], w = norm_a for the first heads_a heads, norm_b for the others;
 //   rotation (inv_freq != null) of the first `dims` numbers by angle_i = float(position) * inv_freq[i]: pair (2i, 2i + 1), or, `halves`,
 //   pair (i, i + dims / 2); (u, v) <- (u cos - v sin, v cos + u sin).  What lies beyond `dims` is not turned.  One rounding at the end.
+// `raw_b` (optional, [T, raw_ld]): the heads_b heads as they come, before norm and rotation, are copied there (values that are the keys
+// as projected).
 #define HNR_WAVES 4
 template <typename T>
 __global__ void __launch_bounds__(HNR_WAVES * TL_WAVE)
 head_norm_rotate_kernel(T* __restrict__ x, int ld, int tokens, int heads_a, int heads_b, int dim, const float* __restrict__ norm_a,
                         const float* __restrict__ norm_b, float eps, const int* __restrict__ positions, const float* __restrict__ inv_freq,
-                        int dims, int halves) {
+                        int dims, int halves, T* __restrict__ raw_b, int raw_ld) {
     __shared__ float sv[HNR_WAVES][LA_MAX_DIM];
     const int wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
     const int heads = heads_a + heads_b;
@@ -548,8 +559,14 @@ head_norm_rotate_kernel(T* __restrict__ x, int ld, int tokens, int heads_a, int 
     float* v = sv[wave];
     const float* w = h < heads_a ? norm_a : norm_b;
     float ss = 0.f;
-    if (live)
-        for (int d = lane; d < dim; d += TL_WAVE) { const float a = to_float(row[d]); v[d] = a; ss = fmaf(a, a, ss); }
+    if (live) {
+        T* raw = (raw_b && h >= heads_a) ? raw_b + (size_t)t * raw_ld + (size_t)(h - heads_a) * dim : nullptr;
+        for (int d = lane; d < dim; d += TL_WAVE) {
+            const T x0 = row[d];
+            if (raw) raw[d] = x0;
+            const float a = to_float(x0); v[d] = a; ss = fmaf(a, a, ss);
+        }
+    }
     ss = wave_sum(ss);
     __syncthreads();
     if (live && w) {
@@ -574,7 +591,8 @@ head_norm_rotate_kernel(T* __restrict__ x, int ld, int tokens, int heads_a, int 
 }
 
 extern "C" int tl_head_norm_rotate(void* x, int ld, int tokens, int heads_a, int heads_b, int dim, const void* norm_a, const void* norm_b, float eps,
-                                   const void* positions, const void* inv_freq, int dims, int halves, int dtype, hipStream_t stream) {
+                                   const void* positions, const void* inv_freq, int dims, int halves, void* raw_b, int raw_ld, int dtype, hipStream_t stream) {
+    TL_REQUIRE(!raw_b || raw_ld >= heads_b * dim, "head_norm_rotate: the rows of the copy are too short");
     TL_REQUIRE(tokens >= 0 && heads_a >= 0 && heads_b >= 0 && heads_a + heads_b > 0 && dim > 0 && dim <= LA_MAX_DIM && ld >= (heads_a + heads_b) * dim,
                "head_norm_rotate: bad sizes");
     TL_REQUIRE(!inv_freq || (positions && dims > 0 && dims % 2 == 0 && dims <= dim), "head_norm_rotate: a rotation over %d of %d numbers", dims, dim);
@@ -584,10 +602,10 @@ extern "C" int tl_head_norm_rotate(void* x, int ld, int tokens, int heads_a, int
     const int grid = (int)((items + HNR_WAVES - 1) / HNR_WAVES);
     if (dtype == TL_DT_F32)
         head_norm_rotate_kernel<float><<<grid, HNR_WAVES * TL_WAVE, 0, stream>>>((float*)x, ld, tokens, heads_a, heads_b, dim, (const float*)norm_a,
-            (const float*)norm_b, eps, (const int*)positions, (const float*)inv_freq, dims, halves);
+            (const float*)norm_b, eps, (const int*)positions, (const float*)inv_freq, dims, halves, (float*)raw_b, raw_ld);
     else if (dtype == TL_DT_BF16)
         head_norm_rotate_kernel<bf16_t><<<grid, HNR_WAVES * TL_WAVE, 0, stream>>>((bf16_t*)x, ld, tokens, heads_a, heads_b, dim, (const float*)norm_a,
-            (const float*)norm_b, eps, (const int*)positions, (const float*)inv_freq, dims, halves);
+            (const float*)norm_b, eps, (const int*)positions, (const float*)inv_freq, dims, halves, (bf16_t*)raw_b, raw_ld);
     else TL_REQUIRE(false, "head_norm_rotate: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("head_norm_rotate");
     return TL_OK;

@@ -292,31 +292,41 @@ extern "C" int tl_mlstm_scan(const void* qkv, int ld, int k_off, int v_off, cons
 // ------------------------------------------------------------------ gated per-head norm
 // y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * gate(g[t, h, :]) * gain; one wave per token and head.
 // gate 0: sigmoid, 1: silu.  shared_weight: one vector of vdim numbers for all heads.  The rows of g and y may be longer than
-// heads * vdim (views into wider buffers).
+// heads * vdim (views into wider buffers).  gate_first: the gate comes before the norm, y = u / sqrt(mean(u^2) + eps) * weight * gain
+// with u = o * gate(g) (a "head" is then whatever stretch of the row is normed together).
 template <typename T>
 __global__ void gated_head_norm_kernel(const float* __restrict__ o, const T* __restrict__ gate, int gate_ld,
                                        const void* __restrict__ weight, int weight_f32, int shared_weight, float eps,
-                                       T* __restrict__ out, int out_ld, int rows, int heads, int vdim, int gate_kind, float gain) {
+                                       T* __restrict__ out, int out_ld, int rows, int heads, int vdim, int gate_kind, float gain, int gate_first) {
     const int row = blockIdx.x * (blockDim.x / TL_WAVE) + threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
     if (row >= rows) return;
     const int t = row / heads, h = row % heads;
     const float* src = o + (size_t)row * vdim;
+    const T* g = gate + (size_t)t * gate_ld + h * vdim;
     float ss = 0.f;
-    for (int i = lane; i < vdim; i += TL_WAVE) ss = fmaf(src[i], src[i], ss);
+    for (int i = lane; i < vdim; i += TL_WAVE) {
+        float u = src[i];
+        if (gate_first) {
+            const float z = to_float(g[i]);
+            const float s = 1.f / (1.f + expf(-z));
+            u *= gate_kind == 1 ? z * s : s;
+        }
+        ss = fmaf(u, u, ss);
+    }
     ss = wave_sum(ss);
     const float inv = 1.f / sqrtf(ss / (float)vdim + eps);
-    const T* g = gate + (size_t)t * gate_ld + h * vdim;
     T* dst = out + (size_t)t * out_ld + h * vdim;
     const int w0 = shared_weight ? 0 : h * vdim;
     for (int i = lane; i < vdim; i += TL_WAVE) {
         const float z = to_float(g[i]);
         const float s = 1.f / (1.f + expf(-z));
-        dst[i] = from_float<T>(src[i] * inv * load_vec(weight, weight_f32, w0 + i) * (gate_kind == 1 ? z * s : s) * gain);
+        dst[i] = from_float<T>(src[i] * (gate_kind == 1 ? z * s : s) * inv * load_vec(weight, weight_f32, w0 + i) * gain);
     }
 }
 
 extern "C" int tl_gated_head_norm(const void* o, const void* gate, int gate_ld, const void* weight, int weight_f32, int shared_weight, float eps,
-                                  void* out, int out_ld, int tokens, int heads, int vdim, int gate_kind, float gain, int dtype, hipStream_t stream) {
+                                  void* out, int out_ld, int tokens, int heads, int vdim, int gate_kind, float gain, int gate_first, int dtype,
+                                  hipStream_t stream) {
     TL_REQUIRE(tokens >= 0 && heads > 0 && vdim > 0 && gate_ld >= heads * vdim && out_ld >= heads * vdim, "gated_head_norm: bad sizes");
     TL_REQUIRE(gate_kind == 0 || gate_kind == 1, "gated_head_norm: unknown gate %d", gate_kind);
     if (tokens == 0) return TL_OK;
@@ -324,10 +334,10 @@ extern "C" int tl_gated_head_norm(const void* o, const void* gate, int gate_ld, 
     dim3 grid((rows + 3) / 4), block(4 * TL_WAVE);
     if (dtype == TL_DT_F32)
         gated_head_norm_kernel<float><<<grid, block, 0, stream>>>((const float*)o, (const float*)gate, gate_ld, weight, weight_f32, shared_weight, eps,
-                                                                  (float*)out, out_ld, rows, heads, vdim, gate_kind, gain);
+                                                                  (float*)out, out_ld, rows, heads, vdim, gate_kind, gain, gate_first);
     else if (dtype == TL_DT_BF16)
         gated_head_norm_kernel<bf16_t><<<grid, block, 0, stream>>>((const float*)o, (const bf16_t*)gate, gate_ld, weight, weight_f32, shared_weight, eps,
-                                                                   (bf16_t*)out, out_ld, rows, heads, vdim, gate_kind, gain);
+                                                                   (bf16_t*)out, out_ld, rows, heads, vdim, gate_kind, gain, gate_first);
     else TL_REQUIRE(false, "gated_head_norm: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("gated_head_norm");
     return TL_OK;
@@ -492,9 +502,11 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-// DELTA false: the same recurrence without the correction, S <- g S + k v^T and o = S^T q, with one fixed decay per head (`head_decay`)
-// in place of the tokens' gates: the decayed linear attention.
-template <int RPL, int TB, bool DELTA>
+// MODE 1: the delta rule.  MODE 0: the same recurrence without the correction, S <- g S + k v^T and o = S^T q, with one fixed decay per
+// head (`head_decay`) in place of the tokens' gates: the decayed linear attention.  MODE 2: without the correction, with the tokens' own
+// decays and step sizes, S <- g S + k (beta v)^T and o = S^T q + skip v with one skip factor per head (`head_decay` holds them): a
+// selective state-space recurrence (k: the input matrix's row B, q: the output matrix's row C, beta: the step size, v: the input).
+template <int RPL, int TB, int MODE>
 __global__ void __launch_bounds__(256)
 delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates, const float* __restrict__ head_decay,
                   float* __restrict__ state, size_t slot_stride,
@@ -549,13 +561,14 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
                     if (e < ROWS) v = e < dim ? row[q_at + e] : 0.f;
                     else if (e < 2 * ROWS) v = e - ROWS < dim ? row[k_at + e - ROWS] : 0.f;
                     else if (e < 2 * ROWS + DELTA_COLS) v = col0 + e - 2 * ROWS < vdim ? row[v_at + e - 2 * ROWS] : 0.f;
-                    else if (DELTA) v = gates[(size_t)(base + t) * 2 * heads + (e - 2 * ROWS - DELTA_COLS) * heads + head];
+                    else if (MODE != 0) v = gates[(size_t)(base + t) * 2 * heads + (e - 2 * ROWS - DELTA_COLS) * heads + head];
                     else v = e == PER_TOKEN - 1 ? head_decay[head] : 1.f;
                 } else if (e == PER_TOKEN - 1) v = 1.f;        // beyond the request's last token: k = 0, beta = 0 and a decay of 1 leave the state as it is, to the bit
             }
             stage[j] = v;
         }
     };
+    const float skip = MODE == 2 ? head_decay[head] : 0.f;
     fetch(tok0);
     for (int base = tok0; base < tok1; base += tb) {
         const int nb = min(tb, tok1 - base);
@@ -594,17 +607,17 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
                 float a4[4] = {0.f, 0.f, 0.f, 0.f}, b4[4] = {0.f, 0.f, 0.f, 0.f}, c4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int r = 0; r < RPL; ++r) {
-                    if (DELTA) a4[r & 3] = fmaf(S[r], kr[r], a4[r & 3]);
+                    if (MODE == 1) a4[r & 3] = fmaf(S[r], kr[r], a4[r & 3]);
                     b4[r & 3] = fmaf(S[r], qr[r], b4[r & 3]);
                     c4[r & 3] = fmaf(kr[r], qr[r], c4[r & 3]);
                 }
-                const float a = DELTA ? row16_sum((a4[0] + a4[1]) + (a4[2] + a4[3])) : 0.f;
+                const float a = MODE == 1 ? row16_sum((a4[0] + a4[1]) + (a4[2] + a4[3])) : 0.f;
                 const float b = row16_sum((b4[0] + b4[1]) + (b4[2] + b4[3]));
                 const float kq = row16_sum((c4[0] + c4[1]) + (c4[2] + c4[3]));
-                const float u = DELTA ? beta * (vt - g * a) : vt;
+                const float u = MODE == 1 ? beta * (vt - g * a) : (MODE == 2 ? beta * vt : vt);
 #pragma unroll
                 for (int r = 0; r < RPL; ++r) S[r] = fmaf(kr[r], u, g * S[r]);
-                obuf[t] = fmaf(kq, u, g * b);
+                obuf[t] = MODE == 2 ? fmaf(skip, vt, fmaf(kq, u, g * b)) : fmaf(kq, u, g * b);
             }
         }
         if (rg == 0 && col_ok) {
@@ -625,7 +638,7 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
 }
 
 // state: per slot, from its start, heads x [vdim][dim] floats (a head's state column by column).
-template <bool DELTA>
+template <int MODE>
 static int launch_delta_scan(const void* qkv, const void* gates, const void* head_decay, void* state, long slot_stride, const void* slots,
                              const void* req_indptr, void* out, int requests, int heads, int kv_heads, int dim, int vdim, int longest, hipStream_t stream) {
     const int rpl = dim <= 64 ? 4 : dim <= 128 ? 8 : dim <= 192 ? 12 : 16;
@@ -634,7 +647,7 @@ static int launch_delta_scan(const void* qkv, const void* gates, const void* hea
     const size_t smem = sizeof(float) * (size_t)tb * (2 * DELTA_L * rpl + DELTA_COLS + 2);
     dim3 grid((vdim + DELTA_COLS - 1) / DELTA_COLS, heads, requests), block(256);
 #define TL_DELTA_B(R, B)                                                                                                                   \
-    delta_scan_kernel<R, B, DELTA><<<grid, block, smem, stream>>>((const float*)qkv, (const float*)gates, (const float*)head_decay, (float*)state, \
+    delta_scan_kernel<R, B, MODE><<<grid, block, smem, stream>>>((const float*)qkv, (const float*)gates, (const float*)head_decay, (float*)state, \
                                                            (size_t)slot_stride, (const int*)slots, (const int*)req_indptr, (float*)out, heads, kv_heads, dim, vdim)
 #define TL_DELTA(R)                        \
     if (tb == 1) TL_DELTA_B(R, 1);         \
@@ -656,7 +669,7 @@ extern "C" int tl_delta_scan(const void* qkv, const void* gates, void* state, lo
     TL_REQUIRE(slot_stride >= (long)heads * dim * vdim, "delta_scan: the state rows are too short");
     TL_REQUIRE(requests <= 65535 && heads <= 65535, "delta_scan: too many requests or heads for one launch");
     if (requests == 0) return TL_OK;
-    launch_delta_scan<true>(qkv, gates, nullptr, state, slot_stride, slots, req_indptr, out, requests, heads, kv_heads, dim, vdim, longest, stream);
+    launch_delta_scan<1>(qkv, gates, nullptr, state, slot_stride, slots, req_indptr, out, requests, heads, kv_heads, dim, vdim, longest, stream);
     TL_CHECK_LAUNCH("delta_scan");
     return TL_OK;
 }
@@ -671,8 +684,87 @@ extern "C" int tl_decay_scan(const void* qkv, const void* decay, void* state, lo
     TL_REQUIRE(slot_stride >= (long)heads * dim * vdim, "decay_scan: the state rows are too short");
     TL_REQUIRE(requests <= 65535 && heads <= 65535, "decay_scan: too many requests or heads for one launch");
     if (requests == 0) return TL_OK;
-    launch_delta_scan<false>(qkv, nullptr, decay, state, slot_stride, slots, req_indptr, out, requests, heads, heads, dim, vdim, longest, stream);
+    launch_delta_scan<0>(qkv, nullptr, decay, state, slot_stride, slots, req_indptr, out, requests, heads, heads, dim, vdim, longest, stream);
     TL_CHECK_LAUNCH("decay_scan");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ selective state-space recurrence (Mamba-2)
+// Per head S <- decay S + dt B x^T (S: state x vdim), y = S^T C + D x, with B and C shared by the heads of a group.  qkv float [T, 2 * groups *
+// state + heads * vdim] as selective_prepare leaves it (C, B, x), gates float [T, 2 * heads] (dt, decay), skip float [heads] (D); the
+// state as the delta rule's ([vdim][state] per head), out float [T, heads * vdim].
+extern "C" int tl_selective_scan(const void* qkv, const void* gates, const void* skip, void* state, long slot_stride, const void* slots,
+                                 const void* req_indptr, void* out, int requests, int heads, int groups, int dim, int vdim, int longest, hipStream_t stream) {
+    TL_REQUIRE(requests >= 0 && heads > 0 && groups > 0 && heads % groups == 0 && dim > 0 && vdim > 0 && gates && skip, "selective_scan: bad sizes");
+    TL_REQUIRE(dim <= DELTA_L * 16, "selective_scan: built for states of up to %d numbers per column, got %d", DELTA_L * 16, dim);
+    TL_REQUIRE(slot_stride >= (long)heads * dim * vdim, "selective_scan: the state rows are too short");
+    TL_REQUIRE(requests <= 65535 && heads <= 65535, "selective_scan: too many requests or heads for one launch");
+    if (requests == 0) return TL_OK;
+    launch_delta_scan<2>(qkv, gates, skip, state, slot_stride, slots, req_indptr, out, requests, heads, groups, dim, vdim, longest, stream);
+    TL_CHECK_LAUNCH("selective_scan");
+    return TL_OK;
+}
+
+// What that recurrence reads, made from the projection of the step's tokens.  proj [T, ld] holds per token, from column x_off on, the
+// `channels` = inner + 2 * groups * state convolved channels [x | B | C] and after them `heads` raw step sizes.  Channel c at the request's
+// i-th token of the step: y = silu(bias[c] + sum_j w[c][j] * in[i - (taps - 1) + j][c]) with in[i'] the projection of the step's token
+// i' >= 0, else tail[taps - 1 + i'][c] (the slot's last taps - 1 inputs from before the step; zero for a new request).  y goes to qkv
+// float [T, channels] in the order the recurrence reads: C, B, x.  gates float [T, 2 * heads] receives dt = softplus(raw + dt_bias) and
+// decay = exp(-exp(a_log) * dt).  One thread per token and channel (or head).
+template <typename T>
+__global__ void __launch_bounds__(256)
+selective_prepare_kernel(const T* __restrict__ proj, int ld, int x_off, const float* __restrict__ conv_w, const float* __restrict__ conv_b,
+                         float* __restrict__ gates, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+                         const float* __restrict__ state, size_t slot_stride, size_t tail_off, const int* __restrict__ slots,
+                         const int* __restrict__ req_indptr, const int* __restrict__ token_req, float* __restrict__ qkv, int heads, int inner,
+                         int gn, int taps) {
+    const int t = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+    const int channels = inner + 2 * gn;
+    if (c >= channels + heads) return;
+    const T* row = proj + (size_t)t * ld + x_off;
+    if (c >= channels) {
+        const int h = c - channels;
+        const float dt = softplus_f(to_float(row[c]) + dt_bias[h]);
+        gates[(size_t)t * 2 * heads + h] = dt;
+        gates[(size_t)t * 2 * heads + heads + h] = expf(-expf(a_log[h]) * dt);
+        return;
+    }
+    const int req = token_req[t];
+    const int i = t - req_indptr[req];
+    const float* tail = state + (size_t)slots[req] * slot_stride + tail_off;
+    float acc = conv_b[c];
+    for (int j = 0; j < taps; ++j) {
+        const int back = i - (taps - 1) + j;
+        const float xv = back >= 0 ? to_float(proj[(size_t)(t - i + back) * ld + x_off + c]) : tail[(size_t)(taps - 1 + back) * channels + c];
+        acc = fmaf(conv_w[(size_t)c * taps + j], xv, acc);
+    }
+    const int to = c < inner ? 2 * gn + c : (c < inner + gn ? gn + (c - inner) : c - inner - gn);
+    qkv[(size_t)t * channels + to] = silu_f(acc);
+}
+
+extern "C" int tl_selective_prepare(const void* proj, int ld, int x_off, const void* conv_w, const void* conv_b, void* gates, const void* a_log,
+                                    const void* dt_bias, void* state, long slot_stride, long tail_off, const void* slots, const void* req_indptr,
+                                    const void* token_req, void* qkv, int tokens, int requests, int heads, int inner, int gn, int taps, int dtype,
+                                    hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && requests >= 0 && heads > 0 && inner > 0 && gn > 0 && x_off >= 0, "selective_prepare: bad sizes");
+    TL_REQUIRE(taps >= 1 && taps <= DELTA_MAX_TAPS, "selective_prepare: 1 to %d taps are built, not %d", DELTA_MAX_TAPS, taps);
+    const int channels = inner + 2 * gn;
+    TL_REQUIRE(ld >= x_off + channels + heads && tail_off >= 0 && slot_stride >= tail_off + (long)(taps - 1) * channels, "selective_prepare: rows or state too short");
+    TL_REQUIRE(dtype == TL_DT_F32 || dtype == TL_DT_BF16, "selective_prepare: unknown dtype %d", dtype);
+    TL_REQUIRE(requests <= 65535 && (channels + heads + 255) / 256 <= 65535, "selective_prepare: too many requests or channels for one launch");
+    if (tokens == 0 || requests == 0) return TL_OK;
+    dim3 grid(tokens, (channels + heads + 255) / 256), block(256);
+    dim3 tgrid((channels + 255) / 256, requests), tblock(256);
+#define TL_SP(T)                                                                                                                                  \
+    selective_prepare_kernel<T><<<grid, block, 0, stream>>>((const T*)proj, ld, x_off, (const float*)conv_w, (const float*)conv_b, (float*)gates,     \
+        (const float*)a_log, (const float*)dt_bias, (const float*)state, (size_t)slot_stride, (size_t)tail_off, (const int*)slots,               \
+        (const int*)req_indptr, (const int*)token_req, (float*)qkv, heads, inner, gn, taps);                                                      \
+    TL_CHECK_LAUNCH("selective_prepare");                                                                                                         \
+    if (taps > 1) delta_tail_kernel<T><<<tgrid, tblock, 0, stream>>>((const T*)proj + x_off, ld, (float*)state, (size_t)slot_stride, (size_t)tail_off, \
+                                                                     (const int*)slots, (const int*)req_indptr, channels, taps)
+    if (dtype == TL_DT_F32) { TL_SP(float); } else { TL_SP(bf16_t); }
+#undef TL_SP
+    TL_CHECK_LAUNCH("selective_tail");
     return TL_OK;
 }
 

@@ -25,6 +25,8 @@ _libs: dict[str, ctypes.CDLL] = {}
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
+GATE_ACTIVATIONS = {"silu": 0, "relu": 1}      # the activation of a gated feed-forward's gate
+
 
 def _lib(name: str) -> ctypes.CDLL:
     lib = _libs.get(name)
@@ -141,6 +143,21 @@ def embedding(token_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, s
                                  c_int(T), c_int(H), c_int(V), c_float(scale), _ptr(positions if pos_rows else None),
                                  _ptr(pos_table), c_int(_dt(pos_table, "position table") if pos_rows else 0), c_int(pos_rows),
                                  c_int(copies), _stream()))
+
+
+def embedding_norm(token_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float, weight: torch.Tensor, eps: float) -> None:
+    """``out[t] = r / sqrt(mean(r^2) + eps) * weight`` with ``r = float(table[token_ids[t]]) * scale``: ``out`` is the 32-bit residual ``[T, H]``,
+    ``weight`` float32 ``[H]``."""
+    T = token_ids.numel()
+    V, H = table.shape
+    _i32(token_ids, "embedding ids", T)
+    if out.shape != (T, H) or out.dtype != torch.float32 or not out.is_contiguous() or not table.is_contiguous():
+        raise KernelError(f"embedding_norm: out must be contiguous float32 [{T}, {H}], got {out.dtype} {tuple(out.shape)}")
+    if weight.dtype != torch.float32 or weight.shape != (H,) or not weight.is_contiguous():
+        raise KernelError(f"embedding_norm: the norm's weight must be contiguous float32 [{H}]")
+    lib = _lib("elementwise")
+    _check(lib, lib.tl_embedding_norm(_ptr(token_ids), _ptr(table), c_int(_dt(table, "embedding table")), _ptr(out), c_int(T), c_int(H), c_int(V),
+                                      c_float(scale), _ptr(weight), c_float(eps), _stream()))
 
 
 def bigram_embedding(token_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float, bigram: torch.Tensor, buckets: int,
@@ -423,19 +440,21 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return torch.stack((g.view(blocks, 32, K), u.view(blocks, 32, K)), dim=1).reshape(blocks * 64, K).contiguous()
 
 
-def linear_swiglu(x: torch.Tensor, gate_up: torch.Tensor, out: torch.Tensor) -> None:
-    """``out = silu(x @ gate.T) * (x @ up.T)`` on the matrix cores with the gate applied to the
-    32-bit accumulators; ``gate_up`` from :func:`interleave_gate_up`, bfloat16 only,
-    ``x [M, K]`` with K a multiple of 8."""
+def linear_swiglu(x: torch.Tensor, gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
+    """``out = act(x @ gate.T) * (x @ up.T)`` on the matrix cores with the gate applied to the
+    32-bit accumulators (``activation``: ``silu`` or ``relu``); ``gate_up`` from :func:`interleave_gate_up`,
+    bfloat16 only, ``x [M, K]`` with K a multiple of 8."""
     M, K = x.shape
     I = out.shape[1]
     if x.dtype != torch.bfloat16 or gate_up.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
         raise KernelError("linear_swiglu: bfloat16 only")
     if gate_up.shape != (-(-I // 32) * 64, K) or out.shape[0] != M or not gate_up.is_contiguous() or x.stride(1) != 1 or out.stride(1) != 1:
         raise KernelError(f"linear_swiglu: shapes x{tuple(x.shape)} w{tuple(gate_up.shape)} out{tuple(out.shape)} do not fit")
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"linear_swiglu: the gate's activation is one of {', '.join(GATE_ACTIVATIONS)}, not {activation!r}")
     lib = _lib("gemm")
     _check(lib, lib.tl_gemm_swiglu(_ptr(x), _ptr(gate_up), _ptr(out), c_int(M), c_int(I), c_int(K),
-                                   c_int(x.stride(0)), c_int(out.stride(0)), _stream()))
+                                   c_int(x.stride(0)), c_int(out.stride(0)), c_int(GATE_ACTIVATIONS[activation]), _stream()))
 
 
 def linear_swiglu_direct_variant(x: torch.Tensor, gate_up: torch.Tensor, out: torch.Tensor, tile_m: int, tile_n: int) -> None:
@@ -810,13 +829,15 @@ def paged_attention_prompt(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Te
                                               c_int(splits), _ptr(part_o), _ptr(part_ml), _ptr(tokens), c_int(count), _stream()))
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
-    """``out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]``."""
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
+    """``out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i]``; ``activation``: ``silu`` or ``relu``."""
     T, I2 = gate_up.shape
     if I2 % 2 or out.shape != (T, I2 // 2) or out.dtype != gate_up.dtype or not out.is_contiguous() or not gate_up.is_contiguous():
         raise KernelError("swiglu: shapes or dtypes do not fit")
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"swiglu: the gate's activation is one of {', '.join(GATE_ACTIVATIONS)}, not {activation!r}")
     lib = _lib("elementwise")
-    _check(lib, lib.tl_swiglu(_ptr(gate_up), _ptr(out), c_int(T), c_int(I2 // 2), c_int(_dt(out, "swiglu")), _stream()))
+    _check(lib, lib.tl_swiglu(_ptr(gate_up), _ptr(out), c_int(T), c_int(I2 // 2), c_int(_dt(out, "swiglu")), c_int(GATE_ACTIVATIONS[activation]), _stream()))
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor | None, keys: torch.Tensor | None, out: torch.Tensor) -> None:
@@ -911,10 +932,12 @@ GATES = {"sigmoid": 0, "silu": 1}
 
 
 def gated_head_norm(o: torch.Tensor, gate_values: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, heads: int, vdim: int,
-                    gate: str = "sigmoid", gain: float = 1.0) -> None:
+                    gate: str = "sigmoid", gain: float = 1.0, gate_first: bool = False) -> None:
     """``out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * weight[h] * gate(gate_values[t, h]) * gain`` per token and head:
     ``o`` float32 ``[T, heads * vdim]``, ``gate_values`` and ``out`` row-strided views ``[T, heads * vdim]`` of one dtype; ``weight``
-    ``[heads * vdim]``, or ``[vdim]``: one vector for all heads; ``gate``: ``sigmoid`` or ``silu``."""
+    ``[heads * vdim]``, or ``[vdim]``: one vector for all heads; ``gate``: ``sigmoid`` or ``silu``.  ``gate_first``: the gate comes before the
+    norm, ``out = u / sqrt(mean(u^2) + eps) * weight * gain`` with ``u = o * gate(gate_values)``; a "head" is whatever stretch of the row is
+    normed together."""
     T = o.shape[0]
     if o.dtype != torch.float32 or o.shape != (T, heads * vdim) or not o.is_contiguous():
         raise KernelError("gated_head_norm: o must be contiguous float32 [T, heads * vdim]")
@@ -925,7 +948,7 @@ def gated_head_norm(o: torch.Tensor, gate_values: torch.Tensor, weight: torch.Te
     lib = _lib("recurrent")
     _check(lib, lib.tl_gated_head_norm(_ptr(o), _ptr(gate_values), c_int(gate_values.stride(0)), _ptr(weight), c_int(wf), c_int(1 if shared else 0),
                                        c_float(eps), _ptr(out), c_int(out.stride(0)), c_int(T), c_int(heads), c_int(vdim), c_int(GATES[gate]),
-                                       c_float(gain), c_int(_dt(out, "gated_head_norm")), _stream()))
+                                       c_float(gain), c_int(1 if gate_first else 0), c_int(_dt(out, "gated_head_norm")), _stream()))
 
 
 # ------------------------------------------------------------- gated delta rule
@@ -1018,6 +1041,69 @@ def decay_scan(qkv: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, slot
                                   c_int(max(1, T - R + 1) if max_new_tokens is None else max_new_tokens), _stream()))
 
 
+def selective_prepare(proj: torch.Tensor, x_off: int, conv_w: torch.Tensor, conv_b: torch.Tensor, gates: torch.Tensor, a_log: torch.Tensor,
+                      dt_bias: torch.Tensor, state: torch.Tensor, tail_off: int, slots: torch.Tensor, req_indptr: torch.Tensor,
+                      token_req: torch.Tensor, qkv: torch.Tensor, heads: int, inner: int, gn: int, taps: int) -> None:
+    """What a selective state-space recurrence reads, made from the projection of the step's tokens.  ``proj [T, >= x_off + channels + heads]``
+    (rows may be strided) holds per token, from column ``x_off`` on, ``channels = inner + 2 * gn`` convolved channels ``[x | B | C]`` and then
+    ``heads`` raw step sizes.  Every channel passes a causal convolution with a bias, ``y[t] = conv_b[c] + sum_j conv_w[c, j] x[t - (taps - 1) +
+    j]``, whose inputs before the step's first token of a request come from the request's slot (``state[slot, tail_off + i * channels + c]``,
+    oldest first), then silu; the result goes to ``qkv`` float32 ``[T, channels]`` in the order ``[C | B | x]``.  ``gates`` float32 ``[T, 2 *
+    heads]`` receives ``dt = softplus(raw + dt_bias)`` and ``exp(-exp(a_log) * dt)``.  Afterwards the slots' tails hold the last ``taps - 1``
+    inputs of every request."""
+    T = proj.shape[0]
+    R = req_indptr.numel() - 1
+    C = inner + 2 * gn
+    if proj.stride(1) != 1 or proj.shape[1] < x_off + C + heads or qkv.dtype != torch.float32 or qkv.shape != (T, C) or not qkv.is_contiguous():
+        raise KernelError("selective_prepare: the projection or the output does not hold the convolved channels")
+    if conv_w.dtype != torch.float32 or conv_w.shape != (C, taps) or not conv_w.is_contiguous() or not 1 <= taps <= DELTA_MAX_TAPS \
+            or conv_b.dtype != torch.float32 or conv_b.shape != (C,) or not conv_b.is_contiguous():
+        raise KernelError(f"selective_prepare: taps must be contiguous float32 [{C}, {taps}] (up to {DELTA_MAX_TAPS} of them) with a bias [{C}]")
+    if gates.dtype != torch.float32 or gates.shape != (T, 2 * heads) or not gates.is_contiguous():
+        raise KernelError(f"selective_prepare: gates must be contiguous float32 [{T}, {2 * heads}]")
+    for v, what in ((a_log, "a_log"), (dt_bias, "dt_bias")):
+        if v.dtype != torch.float32 or v.shape != (heads,) or not v.is_contiguous():
+            raise KernelError(f"selective_prepare: {what} must be contiguous float32 [{heads}]")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < tail_off + (taps - 1) * C:
+        raise KernelError(f"selective_prepare: state {tuple(state.shape)} does not hold the convolutions' tails")
+    _i32(slots, "slots", R)
+    _i32(req_indptr, "req_indptr", R + 1)
+    _i32(token_req, "token_req", T)
+    lib = _lib("recurrent")
+    _check(lib, lib.tl_selective_prepare(_ptr(proj), c_int(proj.stride(0)), c_int(x_off), _ptr(conv_w), _ptr(conv_b), _ptr(gates), _ptr(a_log),
+                                         _ptr(dt_bias), _ptr(state), ctypes.c_long(state.stride(0)), ctypes.c_long(tail_off), _ptr(slots),
+                                         _ptr(req_indptr), _ptr(token_req), _ptr(qkv), c_int(T), c_int(R), c_int(heads), c_int(inner), c_int(gn),
+                                         c_int(taps), c_int(_dt(proj, "selective_prepare")), _stream()))
+
+
+def selective_scan(qkv: torch.Tensor, gates: torch.Tensor, skip: torch.Tensor, state: torch.Tensor, slots: torch.Tensor, req_indptr: torch.Tensor,
+                   out: torch.Tensor, heads: int, groups: int, dim: int, vdim: int, max_new_tokens: int | None = None) -> None:
+    """A selective state-space recurrence over the step's tokens, request by request from the state its slot holds: ``qkv`` float32 ``[T, 2 *
+    groups * dim + heads * vdim]`` as :func:`selective_prepare` left it (C, B, x), ``gates`` float32 ``[T, 2 * heads]`` (dt, decay), ``skip``
+    float32 ``[heads]``; head ``h`` (reading B and C of group ``h // (heads / groups)``) of ``state[slot]`` (float32, ``dim x vdim`` numbers from ``h *
+    dim * vdim`` on, column by column: ``[vdim][dim]``) moves by ``S <- decay S + dt B x^T`` and ``out`` float32 ``[T, heads * vdim]`` receives
+    ``S^T C + skip[h] x``."""
+    T = qkv.shape[0]
+    R = req_indptr.numel() - 1
+    C = 2 * groups * dim + heads * vdim
+    if qkv.dtype != torch.float32 or qkv.shape != (T, C) or not qkv.is_contiguous():
+        raise KernelError(f"selective_scan: qkv must be contiguous float32 [{T}, {C}]")
+    if gates.dtype != torch.float32 or gates.shape != (T, 2 * heads) or not gates.is_contiguous():
+        raise KernelError(f"selective_scan: gates must be contiguous float32 [{T}, {2 * heads}]")
+    if skip.dtype != torch.float32 or skip.shape != (heads,) or not skip.is_contiguous():
+        raise KernelError(f"selective_scan: skip must be contiguous float32 [{heads}]")
+    if out.dtype != torch.float32 or out.shape != (T, heads * vdim) or not out.is_contiguous():
+        raise KernelError(f"selective_scan: out must be contiguous float32 [{T}, {heads * vdim}]")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < heads * dim * vdim or dim > DELTA_MAX_DIM or heads % groups:
+        raise KernelError(f"selective_scan: state {tuple(state.shape)} does not hold {heads} states of {dim} x {vdim} (up to {DELTA_MAX_DIM} rows)")
+    _i32(slots, "slots", R)
+    _i32(req_indptr, "req_indptr", R + 1)
+    lib = _lib("recurrent")
+    _check(lib, lib.tl_selective_scan(_ptr(qkv), _ptr(gates), _ptr(skip), _ptr(state), ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(req_indptr),
+                                      _ptr(out), c_int(R), c_int(heads), c_int(groups), c_int(dim), c_int(vdim),
+                                      c_int(max(1, T - R + 1) if max_new_tokens is None else max_new_tokens), _stream()))
+
+
 def silu_float(x: torch.Tensor, out: torch.Tensor) -> None:
     """``out = silu(float32(x))``: ``x [T, C]`` a row-strided view of either dtype, ``out`` contiguous float32 ``[T, C]``."""
     if x.dim() != 2 or x.stride(1) != 1 or out.dtype != torch.float32 or out.shape != x.shape or not out.is_contiguous():
@@ -1071,7 +1157,7 @@ def local_attention_mfma_fits(dtype: torch.dtype, dim: int, vdim: int, page_size
 def local_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v_plane: torch.Tensor, block_table: torch.Tensor,
                     token_req: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, page_size: int,
                     scale: float, softcap: float = 0.0, chunk: int = 0, window: int = 0, gain: float = 1.0, tiles=None,
-                    sink: torch.Tensor | None = None, pooled=None) -> None:
+                    sink: torch.Tensor | None = None, pooled=None, keep_first: int = 0) -> None:
     """Attention of the step's queries ``q [T, heads * dim]`` over their requests' cached keys and values (which hold the step's own tokens
     already): query head ``i`` reads key/value head ``i // (heads / kv_heads)``; ``score = q . k * scale``, then (``softcap > 0``) ``softcap *
     tanh(score / softcap)``; a query at position ``p`` reads the keys ``j <= p`` with ``j // chunk == p // chunk`` (``chunk > 0``) and ``j > p -
@@ -1080,8 +1166,11 @@ def local_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
     (req_indptr, ctx_lens, tile_req, tile_tok0, number of tiles)`` (tiles of up to 16 consecutive tokens of one request, as a step
     context makes them) runs the matrix-core kernel, where :func:`local_attention_mfma_fits` says it is built.  ``sink`` (float32 ``[heads]``):
     ``exp(sink[head])`` joins the softmax's denominator.  ``pooled = (pk_plane, pv_plane, pool_table, pool)`` (with a window): a query at
-    ``p`` also reads the rows ``0 .. (p - window + 1) // pool - 1`` of these planes (laid out like the tokens', with a block table of their own)."""
+    ``p`` also reads the rows ``0 .. (p - window + 1) // pool - 1`` of these planes (laid out like the tokens', with a block table of their own).
+    ``keep_first`` (with a window, without chunks): a query also reads the keys at the positions ``0 .. keep_first - 1``, wherever it stands."""
     T = q.shape[0]
+    if keep_first < 0 or (keep_first and (window <= 0 or chunk)):
+        raise KernelError("local_attention: kept first tokens stand beside a window, without chunks")
     _check_local_planes("local_attention", k_plane, v_plane, q.dtype, kv_heads, dim, vdim, page_size)
     if sink is not None and (sink.dtype != torch.float32 or sink.shape != (heads,) or not sink.is_contiguous()):
         raise KernelError(f"local_attention: the sink must be contiguous float32 [{heads}]")
@@ -1116,14 +1205,14 @@ def local_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
                                                  _ptr(req_indptr), _ptr(ctx_lens), _ptr(tile_req), _ptr(tile_tok0), c_int(n_tiles), c_int(heads),
                                                  c_int(kv_heads), c_int(dim), c_int(vdim), c_int(page_size), c_float(scale), c_float(softcap),
                                                  c_int(chunk), c_int(window), c_float(gain), *pool_args, c_int(pool_table.shape[1] if pool else 0),
-                                                 c_int(pool), _stream()))
+                                                 c_int(pool), c_int(keep_first), _stream()))
         return
     _i32(token_req, "token_req", T)
     _i32(positions, "positions", T)
     _check(lib, lib.tl_local_attention(_ptr(q), c_int(q.stride(0)), _ptr(out), c_int(out.stride(0)), _ptr(k_plane), _ptr(v_plane), c_int(k_plane.shape[0]),
                                        _ptr(block_table), c_int(block_table.stride(0)), c_int(block_table.shape[1]), _ptr(token_req), _ptr(positions),
                                        c_int(T), c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim), c_int(page_size), c_float(scale),
-                                       c_float(softcap), c_int(chunk), c_int(window), c_float(gain), *pool_args, c_int(pool),
+                                       c_float(softcap), c_int(chunk), c_int(window), c_float(gain), *pool_args, c_int(pool), c_int(keep_first),
                                        c_int(_dt(q, "local_attention")), _stream()))
 
 
@@ -1153,13 +1242,17 @@ def pool_blocks(k_plane: torch.Tensor, v_plane: torch.Tensor, block_table: torch
 
 
 def head_norm_rotate(x: torch.Tensor, heads_a: int, heads_b: int, dim: int, norm_a: torch.Tensor | None, norm_b: torch.Tensor | None, eps: float,
-                     positions: torch.Tensor | None, inv_freq: torch.Tensor | None, dims: int, halves: bool) -> None:
+                     positions: torch.Tensor | None, inv_freq: torch.Tensor | None, dims: int, halves: bool,
+                     raw_b: torch.Tensor | None = None) -> None:
     """In place on ``x [T, (heads_a + heads_b) * dim]`` (a row-strided view: queries, then keys), per token and head, in 32-bit with one rounding:
     a root-mean-square norm over the head's ``dim`` numbers with the weight ``norm_a`` (the first ``heads_a`` heads) or ``norm_b`` (float32
     ``[dim]``; ``None``: no norm), then the rotation of the first ``dims`` numbers by ``float32(position) * inv_freq[i]`` (float32 ``[dims / 2]``;
-    ``None``: no rotation), pairing ``2i`` with ``2i + 1`` or, ``halves``, ``i`` with ``i + dims / 2``."""
+    ``None``: no rotation), pairing ``2i`` with ``2i + 1`` or, ``halves``, ``i`` with ``i + dims / 2``.  ``raw_b [T, heads_b * dim]`` (of ``x``'s
+    dtype, rows may be strided) receives the last ``heads_b`` heads as they come, before norm and rotation."""
     T = x.shape[0]
     heads = heads_a + heads_b
+    if raw_b is not None and (raw_b.dtype != x.dtype or raw_b.shape != (T, heads_b * dim) or raw_b.stride(1) != 1):
+        raise KernelError(f"head_norm_rotate: the copy of the second heads must be [T, {heads_b * dim}] of {x.dtype}")
     if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] != heads * dim or dim > LOCAL_ATTENTION_MAX_DIM:
         raise KernelError(f"head_norm_rotate: x {tuple(x.shape)} is not [T, {heads} heads of {dim}] (up to {LOCAL_ATTENTION_MAX_DIM} numbers a head)")
     for w in (norm_a, norm_b):
@@ -1176,7 +1269,8 @@ def head_norm_rotate(x: torch.Tensor, heads_a: int, heads_b: int, dim: int, norm
     lib = _lib("local_attention")
     _check(lib, lib.tl_head_norm_rotate(_ptr(x), c_int(x.stride(0)), c_int(T), c_int(heads_a), c_int(heads_b), c_int(dim), _ptr(norm_a), _ptr(norm_b),
                                         c_float(eps), _ptr(positions if inv_freq is not None else None), _ptr(inv_freq), c_int(dims if inv_freq is not None else 0),
-                                        c_int(1 if halves else 0), c_int(_dt(x, "head_norm_rotate")), _stream()))
+                                        c_int(1 if halves else 0), _ptr(raw_b), c_int(raw_b.stride(0) if raw_b is not None else 0),
+                                        c_int(_dt(x, "head_norm_rotate")), _stream()))
 
 
 # ------------------------------------------------------------- attention over a cached latent
@@ -1201,14 +1295,15 @@ def latent_attention_mfma_fits(dtype: torch.dtype, heads: int, rank: int, rot: i
     return dtype == torch.bfloat16 and bool(_lib("latent").tl_latent_attention_mfma_fits(c_int(rank), c_int(rot), c_int(heads * (rank + rot))))
 
 
-def latent_prepare(down: torch.Tensor, q_rank: int, rank: int, rot: int, rot_dims: int, wq: torch.Tensor, wkv: torch.Tensor, eps: float,
-                   positions: torch.Tensor, inv_freq: torch.Tensor, cq: torch.Tensor, token_req: torch.Tensor | None = None,
+def latent_prepare(down: torch.Tensor, q_rank: int, kv_off: int, rank: int, rot: int, rot_dims: int, wq: torch.Tensor | None, wkv: torch.Tensor,
+                   eps: float, positions: torch.Tensor, inv_freq: torch.Tensor, cq: torch.Tensor | None, token_req: torch.Tensor | None = None,
                    block_table: torch.Tensor | None = None, plane: torch.Tensor | None = None, page_size: int = 0) -> None:
-    """From the fused down-projection ``down [T, q_rank + rank + rot]``: ``cq = rmsnorm(down[:, :q_rank]) * wq`` and, with a
-    plane ``[pages, 1, page, rank + rot]``, the token's cache row ``[rmsnorm(down[:, q_rank:q_rank + rank]) * wkv, the last
-    rot numbers with the first rot_dims of them turned in pairs by the token's position]``."""
+    """From the fused first projection ``down [T, >= kv_off + rank + rot]``: ``cq = rmsnorm(down[:, :q_rank]) * wq`` (``q_rank`` 0: no query
+    latent, ``wq`` and ``cq`` ``None``) and, with a plane ``[pages, 1, page, rank + rot]``, the token's cache row ``[rmsnorm(down[:, kv_off:kv_off +
+    rank]) * wkv, the next rot numbers with the first rot_dims of them turned in pairs by the token's position]``."""
     T = down.shape[0]
-    if down.stride(1) != 1 or down.shape[1] < q_rank + rank + rot or cq.shape != (T, q_rank) or cq.dtype != down.dtype or not cq.is_contiguous():
+    if down.stride(1) != 1 or kv_off < q_rank or down.shape[1] < kv_off + rank + rot or (q_rank == 0) != (cq is None) or (q_rank == 0) != (wq is None) \
+            or (cq is not None and (cq.shape != (T, q_rank) or cq.dtype != down.dtype or not cq.is_contiguous())):
         raise KernelError("latent_prepare: shapes do not fit")
     _i32(positions, "positions", T)
     if inv_freq.dtype != torch.float32 or inv_freq.numel() != rot_dims // 2 or rot_dims % 2 or rot_dims > rot:
@@ -1221,7 +1316,7 @@ def latent_prepare(down: torch.Tensor, q_rank: int, rank: int, rot: int, rot_dim
         if plane.dtype != down.dtype or plane.dim() != 4 or tuple(plane.shape[1:]) != (1, page_size, rank + rot) or not plane.is_contiguous():
             raise KernelError(f"latent_prepare: plane {tuple(plane.shape)} {plane.dtype} is not [pages, 1, {page_size}, {rank + rot}] {down.dtype}")
     lib = _lib("latent")
-    _check(lib, lib.tl_latent_prepare(_ptr(down), c_int(down.stride(0)), c_int(q_rank), c_int(rank), c_int(rot), c_int(rot_dims),
+    _check(lib, lib.tl_latent_prepare(_ptr(down), c_int(down.stride(0)), c_int(q_rank), c_int(kv_off), c_int(rank), c_int(rot), c_int(rot_dims),
                                       _ptr(wq), c_int(_vec(wq, q_rank, "query latent norm")), _ptr(wkv), c_int(_vec(wkv, rank, "latent norm")),
                                       c_float(eps), _ptr(positions), _ptr(inv_freq), _ptr(token_req), _ptr(block_table), c_int(bt_stride),
                                       _ptr(plane), c_int(page_size), _ptr(cq), c_int(T), c_int(_dt(down, "latent_prepare")), _stream()))
@@ -1248,14 +1343,17 @@ def rotate_pairs(src: torch.Tensor, src_head: int, src_off: int, dst: torch.Tens
 def latent_attention(q: torch.Tensor, out: torch.Tensor, plane: torch.Tensor, block_table: torch.Tensor, req_indptr: torch.Tensor | None,
                      ctx_lens: torch.Tensor, tile_req: torch.Tensor | None, tile_tok0: torch.Tensor | None, num_tiles: int,
                      tile_tokens: int, heads: int, rank: int, rot: int, page_size: int, scale: float, sink: torch.Tensor | None,
-                     splits: int = 1, general: bool = False, max_new_tokens: int | None = None) -> None:
+                     splits: int = 1, general: bool = False, max_new_tokens: int | None = None, window: int = 0,
+                     gate: torch.Tensor | None = None) -> None:
     """Causal attention of the step's tokens over their requests' cached rows ``plane [pages, 1, page, rank + rot]``: ``q [T,
     heads * (rank + rot)]`` holds per head the query brought into the cache row's shape, a score is the dot product of the two
     times ``scale``, the softmax's denominator also holds ``exp(sink[head])`` (float32 ``[heads]``; ``None``: no sink), and ``out
     [T, heads * rank]`` receives the weighted sums of the rows' first ``rank`` numbers.  ``tile_req = tile_tok0 = None``: every
     request brings one token.  ``splits``: work-groups that share a tile's keys (merged afterwards).  bfloat16 at sizes that
     :func:`latent_attention_mfma_fits` runs on the matrix cores (``general=True`` forces the general kernel); ``max_new_tokens``:
-    the most tokens a request brings in this step (default: ``tile_tokens``), by which the matrix-core kernel sizes its work-groups."""
+    the most tokens a request brings in this step (default: ``tile_tokens``), by which the matrix-core kernel sizes its work-groups.
+    ``window > 0``: a query reads its last ``window`` keys only, itself included.  ``gate [T, >= heads]`` (of ``q``'s dtype, rows may be
+    strided): head ``n``'s output of token ``t`` is multiplied by ``sigmoid(gate[t, n])``."""
     T = q.shape[0]
     D = rank + rot
     if q.stride(1) != 1 or q.shape[1] < heads * D or out.shape != (T, heads * rank) or not out.is_contiguous() or out.dtype != q.dtype:
@@ -1277,6 +1375,8 @@ def latent_attention(q: torch.Tensor, out: torch.Tensor, plane: torch.Tensor, bl
             raise KernelError("latent_attention: tile arrays shorter than the number of tiles")
     if sink is not None and (sink.dtype != torch.float32 or sink.numel() != heads or not sink.is_contiguous()):
         raise KernelError("latent_attention: sink must be float32 [heads]")
+    if window < 0 or (gate is not None and (gate.dtype != q.dtype or gate.dim() != 2 or gate.shape[0] != T or gate.shape[1] < heads or gate.stride(1) != 1)):
+        raise KernelError("latent_attention: a window is not negative, and a gate is [T, >= heads] of the queries' dtype")
     splits = max(1, min(splits, SPLIT_SCRATCH_BYTES // (T * heads * (rank + 2) * 4)))
     part_o = part_ml = None
     if splits > 1:
@@ -1287,7 +1387,8 @@ def latent_attention(q: torch.Tensor, out: torch.Tensor, plane: torch.Tensor, bl
                                         _ptr(req_indptr), _ptr(ctx_lens), _ptr(tile_req), _ptr(tile_tok0), c_int(num_tiles), c_int(T),
                                         c_int(tile_tokens), c_int(heads), c_int(rank), c_int(rot), c_int(page_size), c_float(scale),
                                         _ptr(sink), c_int(splits), _ptr(part_o), _ptr(part_ml), c_int(_dt(q, "latent_attention")),
-                                        c_int(1 if general else 0), c_int(tile_tokens if max_new_tokens is None else max_new_tokens), _stream()))
+                                        c_int(1 if general else 0), c_int(tile_tokens if max_new_tokens is None else max_new_tokens),
+                                        c_int(window), _ptr(gate), c_int(gate.stride(0) if gate is not None else 0), _stream()))
 
 
 # ------------------------------------------------------------- products over groups, routing
@@ -1331,14 +1432,17 @@ def experts_linear(x: torch.Tensor, slot_token: torch.Tensor | None, weight: tor
                                     c_int(_dt(x, "experts_linear")), c_int(1 if general else 0), _stream()))
 
 
-ROUTER_SCORES = {"chosen": 0, "all": 1}
+ROUTER_SCORES = {"chosen": 0, "all": 1, "sigmoid": 2}
 
 
-def route(logits: torch.Tensor, top: int, scores: str = "chosen", choice_bias: torch.Tensor | None = None):
+def route(logits: torch.Tensor, top: int, scores: str = "chosen", choice_bias: torch.Tensor | None = None, weight_scale: float = 1.0,
+          weight_eps: float = 0.0):
     """The router's choice for every row of float32 ``logits [T, experts]`` and the sort of the (token, choice) pairs by expert.
     ``scores="chosen"``: the ``top`` largest logits are chosen and weighed by the softmax over those alone; ``"all"``: the scores are the
     softmax over all logits, the ``top`` largest of score (+ ``choice_bias [experts]``, float32, which enters the choice only) are chosen
-    and weighed by their scores as they are.  The lower index wins a tie.  Returns ``(weights [T, top] float32, offsets [experts + 1],
+    and weighed by their scores as they are; ``"sigmoid"``: the scores are the logits' sigmoids, the choice goes by score (+ ``choice_bias``)
+    and the weights are the chosen scores divided by their sum plus ``weight_eps``.  All weights are multiplied by ``weight_scale``.  The
+    lower index wins a tie.  Returns ``(weights [T, top] float32, offsets [experts + 1],
     slot_token [T * top], pair_slot [T * top])``, all on the GPU: expert ``e`` owns the slots ``offsets[e] .. offsets[e + 1] - 1``, slot
     ``s`` reads token ``slot_token[s]``, and the output row of token ``t``'s ``j``-th choice is ``pair_slot[t * top + j]``."""
     T, E = logits.shape
@@ -1351,14 +1455,15 @@ def route(logits: torch.Tensor, top: int, scores: str = "chosen", choice_bias: t
     weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
     lib = _lib("experts")
     _check(lib, lib.tl_route(_ptr(logits), c_int(T), c_int(E), c_int(top), c_int(ROUTER_SCORES[scores]), _ptr(choice_bias), _ptr(chosen), _ptr(weights),
-                             _ptr(offsets), _ptr(slot_token), _ptr(pair_slot), _stream()))
+                             _ptr(offsets), _ptr(slot_token), _ptr(pair_slot), c_float(weight_scale), c_float(weight_eps), _stream()))
     return weights, offsets, slot_token, pair_slot
 
 
-def combine(y: torch.Tensor, pair_slot: torch.Tensor, weights: torch.Tensor, out: torch.Tensor, identity=None) -> None:
+def combine(y: torch.Tensor, pair_slot: torch.Tensor, weights: torch.Tensor, out: torch.Tensor, identity=None,
+            addend: torch.Tensor | None = None) -> None:
     """``out[t] = sum_j weights[t, j] * y[pair_slot[t * top + j]]``, summed in 32-bit in the order of the choices.  ``identity = (x,
     offsets, experts)``: a pair whose slot is ``offsets[experts]`` or later chose an expert without tensors, and ``x[t]`` stands in for
-    its row of ``y``."""
+    its row of ``y``.  ``addend [T, W]`` (a shared expert's output) is added last, in 32-bit, before the one rounding."""
     T, top = weights.shape
     W = out.shape[1]
     if y.shape != (T * top, W) or out.shape[0] != T or y.dtype != out.dtype or not y.is_contiguous() or not out.is_contiguous() \
@@ -1372,9 +1477,11 @@ def combine(y: torch.Tensor, pair_slot: torch.Tensor, weights: torch.Tensor, out
         if x.shape != (T, W) or x.dtype != out.dtype or not x.is_contiguous():
             raise KernelError("combine: the input that stands in for identity experts does not fit")
         _i32(offsets, "offsets", experts + 1)
+    if addend is not None and (addend.shape != (T, W) or addend.dtype != out.dtype or not addend.is_contiguous()):
+        raise KernelError("combine: the addend does not fit the output")
     lib = _lib("experts")
     _check(lib, lib.tl_combine(_ptr(y), _ptr(pair_slot), _ptr(weights), _ptr(out), _ptr(x), _ptr(offsets), c_int(experts), c_int(T), c_int(top),
-                               c_int(W), c_int(_dt(out, "combine")), _stream()))
+                               c_int(W), _ptr(addend), c_int(_dt(out, "combine")), _stream()))
 
 
 def activation(x: torch.Tensor, kind: str) -> None:

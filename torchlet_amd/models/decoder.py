@@ -33,6 +33,10 @@ class DecoderModel:
         self.position_table: torch.Tensor | None = None
         self.bigram_table: torch.Tensor | None = None
         self.keeps_embedding = any(e.add_embedding for e in spec.order)
+        self.embed_norm = NORMS.build(spec.embed_norm, dtype, self.device) if spec.embed_norm is not None else None
+        if self.embed_norm is not None and (not hasattr(self.embed_norm, "embed") or spec.bigram is not None or spec.position_table_name
+                                            or spec.streams or self.keeps_embedding):
+            raise ValueError("a norm on the embedding needs a norm that makes the normed rows itself, over one plain residual of token rows alone")
         if (spec.bigram is not None or self.keeps_embedding) and spec.streams:
             raise ValueError("a bigram embedding or an embedding that enters the stream again runs over one plain residual")
         if spec.bigram is not None and spec.position_table_name:
@@ -51,6 +55,9 @@ class DecoderModel:
                 specs[join_name(s.layer_name(i), k)] = v
         for k, v in self.final_norm.weight_specs().items():
             specs[join_name(s.final_norm_name, k)] = v
+        if self.embed_norm is not None:
+            for k, v in self.embed_norm.weight_specs().items():
+                specs[join_name(s.embed_norm_name, k)] = v
         # a tied head is the embedding matrix; a checkpoint may still carry a copy of it
         specs[join_name(s.head_name, s.weight_suffix)] = WeightSpec((s.vocab_size, s.hidden), optional=s.tie_head)
         if s.head_bias:
@@ -67,6 +74,8 @@ class DecoderModel:
         for i, block in enumerate(self.blocks):      # (`tensors` may read from disk on access: each name is touched once)
             block.load_weights(under(tensors, s.layer_name(i)))
         self.final_norm.load_weights(under(tensors, s.final_norm_name))
+        if self.embed_norm is not None:      # (its name may lie below the embedding's: the tensor is asked for by its full name)
+            self.embed_norm.load_weights({k: tensors[join_name(s.embed_norm_name, k)] for k in self.embed_norm.weight_specs()})
         if s.tie_head:
             self.head = self.embed
         else:
@@ -94,6 +103,8 @@ class DecoderModel:
         for b in self.blocks:
             yield from b.parts()
         yield from self.final_norm.parts()
+        if self.embed_norm is not None:
+            yield from self.embed_norm.parts()
 
     def graph_safe(self) -> bool:
         """Every part of every block (and the final norm) says that it runs from device-side values only,
@@ -122,6 +133,8 @@ class DecoderModel:
         if big is not None:
             ops.bigram_embedding(ctx.token_ids, self.embed, residual, self.spec.embed_scale, self.bigram_table, big.buckets, big.mul_prev,
                                  big.mul_cur, ctx.token_req, ctx.req_indptr, ctx.positions, ctx.slots, caches[len(self.spec.order)].state)
+        elif self.embed_norm is not None:
+            self.embed_norm.embed(ctx.token_ids, self.embed, residual, self.spec.embed_scale)
         else:
             ops.embedding(ctx.token_ids, self.embed, residual, self.spec.embed_scale,
                           *((ctx.positions, self.position_table) if self.position_table is not None else ()))

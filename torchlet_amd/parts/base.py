@@ -166,7 +166,8 @@ class PagedNeed:
     keys of its own chunk of ``chunk`` positions (counted from position 0), so pages that lie wholly before the chunk of the next
     position are kept no longer.  ``stride``: the planes hold one row for every ``stride`` positions (row ``p // stride``: a summary of a
     block of tokens), so a page of them spans ``stride`` times as many positions.  A mixer that keeps rows at two rates (tokens inside
-    a window, summaries of what lies before it) declares two needs, each a group of its own."""
+    a window, summaries of what lies before it) declares two needs, each a group of its own.  ``keep_first``: beside a window, the first
+    ``keep_first`` positions of a sequence are read by every later query, so the pages that hold them stay with the request."""
     num_heads: int
     head_dim: int
     window: int | None = None
@@ -174,6 +175,7 @@ class PagedNeed:
     dtype: torch.dtype | None = None
     chunk: int | None = None
     stride: int = 1
+    keep_first: int = 0
 
     @property
     def bounded(self) -> bool:
@@ -335,6 +337,8 @@ class StagedMixer(Mixer):
     mix_width: int = 0
     w_in: torch.Tensor | None = None
     w_o: torch.Tensor | None = None
+    b_in: torch.Tensor | None = None      # biases of the two projections (a mixer that stands alone may have them; branches of a
+    b_o: torch.Tensor | None = None       # mixer that stacks several projections into one may not)
 
     def mix(self, proj: torch.Tensor, h: torch.Tensor, ctx, cache, out: torch.Tensor, gain: float = 1.0) -> None:
         """``proj [T, in_width]`` (a row-strided view of ``h @ w_in.T``) and ``h`` itself (for what the mixer projects on its own,
@@ -345,21 +349,21 @@ class StagedMixer(Mixer):
         from ..kernels import ops
         T = h.shape[0]
         proj = torch.empty((T, self.in_width), dtype=self.dtype, device=h.device)
-        ops.linear(h, self.w_in, None, proj)
+        ops.linear(h, self.w_in, self.b_in, proj)
         mixed = torch.empty((T, self.mix_width), dtype=self.dtype, device=h.device)
         self.mix(proj, h, ctx, cache, mixed)
-        return project_out(mixed, self.w_o, self.dtype)
+        return project_out(mixed, self.w_o, self.dtype, self.b_o)
 
 
-def project_out(mixed: torch.Tensor, w_o: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
-    """A mixer's output projection ``[T, hidden]``, or (few rows against a narrow matrix, bfloat16) float32 slabs of partial sums
+def project_out(mixed: torch.Tensor, w_o: torch.Tensor, dtype: torch.dtype, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """A mixer's output projection ``[T, hidden]``, or (few rows against a narrow matrix, bfloat16, no bias) float32 slabs of partial sums
     ``[P, T, hidden]`` that the next norm adds up."""
     from ..kernels import ops
     T, hidden = mixed.shape[0], w_o.shape[0]
-    if dtype == torch.bfloat16 and mixed.shape[1] % 64 == 0 and ops.linear_partials_pay(T, hidden, mixed.shape[1]):
+    if bias is None and dtype == torch.bfloat16 and mixed.shape[1] % 64 == 0 and ops.linear_partials_pay(T, hidden, mixed.shape[1]):
         return ops.linear_partials(mixed, w_o)
     out = torch.empty((T, hidden), dtype=dtype, device=mixed.device)
-    ops.linear(mixed, w_o, None, out)
+    ops.linear(mixed, w_o, bias, out)
     return out
 
 

@@ -20,7 +20,7 @@ import torch
 
 from ..config.base import ConfigError
 from ..kernels import ops
-from .base import FEED_FORWARDS, KEEP_COMPUTE, KEEP_FLOAT32, FeedForward, WeightSpec
+from .base import FEED_FORWARDS, KEEP_COMPUTE, KEEP_FLOAT32, FeedForward, WeightSpec, join_name, under
 
 
 def _activation(name: str) -> str:
@@ -76,16 +76,25 @@ class RoutedExperts(FeedForward):
         self.outputs = self.experts + self.identity          # of the router
         if not 0 < spec.top <= self.outputs:
             raise ConfigError(f"a router picks between 1 and all of its experts, not {spec.top} of {self.outputs}")
-        if spec.scores not in ("chosen", "all"):
-            raise ConfigError(f"a router's scores are the softmax over the 'chosen' logits or over 'all', not {spec.scores!r}")
+        if spec.scores not in ops.ROUTER_SCORES:
+            raise ConfigError(f"a router's scores are the softmax over the 'chosen' logits or over 'all', or their 'sigmoid', not {spec.scores!r}")
+        # one more feed-forward that every token passes, added to the weighted sum (any registered kind that returns a whole tensor)
+        self.shared = FEED_FORWARDS.build(spec.shared, dtype, device) if spec.shared is not None else None
         self.act = _activation(spec.activation + "_pairs" if spec.gated else spec.activation)
         self.w_router = self.b_router = self.correction = self.w_up = self.w_down = None
 
     def kernel_libraries(self):
         return ["experts"]
 
+    def parts(self):
+        yield self
+        if self.shared is not None:
+            yield from self.shared.parts()
+
     def weight_specs(self):
         specs = {"router": WeightSpec((self.outputs, self.hidden))}
+        if self.shared is not None:
+            specs.update({join_name("shared", k): v for k, v in self.shared.weight_specs().items()})
         if self.spec.router_bias:
             specs["router.b"] = WeightSpec((self.outputs,), keep=KEEP_FLOAT32)
         if self.spec.choice_bias:
@@ -107,17 +116,26 @@ class RoutedExperts(FeedForward):
             up = [tensors[f"e{e}.up"] for e in range(self.experts)]
         self.w_up = self._place(torch.stack(up), KEEP_COMPUTE)
         self.w_down = self._place(torch.stack([tensors[f"e{e}.down"] for e in range(self.experts)]), KEEP_COMPUTE)
+        if self.shared is not None:
+            self.shared.load_weights(under(tensors, "shared"))
 
     def forward(self, h, ctx):
         T = h.shape[0]
         logits = torch.empty((T, self.outputs), dtype=torch.float32, device=h.device)
         ops.linear(h, self.w_router, self.b_router, logits)
-        weights, offsets, slot_token, pair_slot = ops.route(logits, self.top, self.spec.scores, self.correction)
+        weights, offsets, slot_token, pair_slot = ops.route(logits, self.top, self.spec.scores, self.correction, float(self.spec.weight_scale),
+                                                            float(self.spec.weight_eps))
         z = torch.empty((T * self.top, self.inter), dtype=self.dtype, device=h.device)
         ops.experts_linear(h, slot_token, self.w_up, offsets, z, self.act)
         y = torch.empty((T * self.top, self.hidden), dtype=self.dtype, device=h.device)
         ops.experts_linear(z, None, self.w_down, offsets, y)
         out = torch.empty((T, self.hidden), dtype=self.dtype, device=h.device)
         # (slots of identity experts lie behind those of the last expert with tensors: their rows of z and y are never written or read)
-        ops.combine(y, pair_slot, weights, out, identity=(h, offsets, self.experts) if self.identity else None)
+        shared = None
+        if self.shared is not None:
+            # (a part that may leave slabs of partial sums for a norm to add up is asked for the whole product)
+            shared = self.shared.forward(h, ctx, whole=True) if getattr(self.shared, "takes_whole", False) else self.shared.forward(h, ctx)
+            if shared.dim() != 2:
+                raise ValueError(f"a shared expert must return one [tokens, hidden] tensor; {type(self.shared).__name__} returned {tuple(shared.shape)}")
+        ops.combine(y, pair_slot, weights, out, identity=(h, offsets, self.experts) if self.identity else None, addend=shared)
         return out

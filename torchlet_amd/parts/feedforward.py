@@ -1,5 +1,6 @@
 """Dense SwiGLU feed-forward: ``down(silu(gate(h)) * up(h))``, no biases
-(/root/reference/src/torchlet/v10_triton_paged_gqa/layer/ffn_swiglu.py:22-59).
+(/root/reference/src/torchlet/v10_triton_paged_gqa/layer/ffn_swiglu.py:22-59).  The gate's activation (``silu`` or ``relu``) and the
+three matrices' names come from the specification.
 
 ``gate_proj`` and ``up_proj`` are put into one matrix at load time so that one matrix
 product reads ``h`` once.  In bfloat16 (hidden a multiple of 8) the two are interleaved in
@@ -11,6 +12,7 @@ from __future__ import annotations
 
 import torch
 
+from ..config.base import ConfigError
 from ..kernels import ops
 from .base import FEED_FORWARDS, KEEP_COMPUTE, FeedForward, LazyNorm, WeightSpec
 
@@ -29,53 +31,57 @@ class SwiGLU(FeedForward):
         super().__init__(spec, dtype, device)
         self.hidden = spec.hidden
         self.inter = spec.intermediate
+        self.act = spec.activation
+        if self.act not in ops.GATE_ACTIVATIONS:
+            raise ConfigError(f"a gated feed-forward's activation is one of {', '.join(ops.GATE_ACTIVATIONS)}, not {self.act!r}")
         self.gate_up: torch.Tensor | None = None
         self.down: torch.Tensor | None = None
 
     def weight_specs(self):
         return {
-            "gate_proj.weight": WeightSpec((self.inter, self.hidden)),
-            "up_proj.weight": WeightSpec((self.inter, self.hidden)),
-            "down_proj.weight": WeightSpec((self.hidden, self.inter)),
+            self.spec.gate_name: WeightSpec((self.inter, self.hidden)),
+            self.spec.up_name: WeightSpec((self.inter, self.hidden)),
+            self.spec.down_name: WeightSpec((self.hidden, self.inter)),
         }
 
     def load_weights(self, tensors):
         self.fused_gate = self.dtype == torch.bfloat16 and self.hidden % 8 == 0
         if self.fused_gate:
-            gate = self._place(tensors["gate_proj.weight"], KEEP_COMPUTE)
-            up = self._place(tensors["up_proj.weight"], KEEP_COMPUTE)
+            gate = self._place(tensors[self.spec.gate_name], KEEP_COMPUTE)
+            up = self._place(tensors[self.spec.up_name], KEEP_COMPUTE)
             self.gate_up = ops.interleave_gate_up(gate, up)
         else:
-            self.gate_up = self._place(torch.cat((tensors["gate_proj.weight"], tensors["up_proj.weight"]), dim=0), KEEP_COMPUTE)
-        self.down = self._place(tensors["down_proj.weight"], KEEP_COMPUTE)
+            self.gate_up = self._place(torch.cat((tensors[self.spec.gate_name], tensors[self.spec.up_name]), dim=0), KEEP_COMPUTE)
+        self.down = self._place(tensors[self.spec.down_name], KEEP_COMPUTE)
 
     takes_lazy_norm = True
+    takes_whole = True          # forward(..., whole=True): one whole [T, hidden] result, never slabs of partial sums (for a caller that is no norm)
 
-    def forward(self, h, ctx):
+    def forward(self, h, ctx, whole: bool = False):
         lazy = h if isinstance(h, LazyNorm) else None
         if lazy is not None:
             # one row: the gate/up kernel makes the norm itself while its first weights arrive
             rms = lazy.rmsnorm()          # the fused kernel makes a root-mean-square norm and no other
-            if self.fused_gate and rms is not None:
+            if self.fused_gate and rms is not None and self.act == "silu":
                 z = torch.empty((1, self.inter), dtype=self.dtype, device=lazy.residual.device)
                 residual_out = torch.empty_like(lazy.residual)
                 if ops.linear_swiglu_normed(lazy.residual, lazy.pending, rms[0], rms[1], residual_out,
                                             self.gate_up, z):
                     lazy.done(residual_out)
-                    return self._down(z, 1)
+                    return self._down(z, 1, whole)
             h = lazy.value()
         T = h.shape[0]
         z = torch.empty((T, self.inter), dtype=self.dtype, device=h.device)
         if self.fused_gate:
-            ops.linear_swiglu(h, self.gate_up, z)
+            ops.linear_swiglu(h, self.gate_up, z, self.act)
         else:
             gu = torch.empty((T, 2 * self.inter), dtype=self.dtype, device=h.device)
             ops.linear(h, self.gate_up, None, gu)
-            ops.swiglu(gu, z)
-        return self._down(z, T)
+            ops.swiglu(gu, z, self.act)
+        return self._down(z, T, whole)
 
-    def _down(self, z, T):
-        if self.dtype == torch.bfloat16 and ops.linear_partials_pay(T, self.hidden, self.inter):
+    def _down(self, z, T, whole=False):
+        if not whole and self.dtype == torch.bfloat16 and ops.linear_partials_pay(T, self.hidden, self.inter):
             # few rows, long K, narrow matrix: split K over work-groups; the next norm adds the slabs up
             return ops.linear_partials(z, self.down)
         y = torch.empty((T, self.hidden), dtype=self.dtype, device=z.device)

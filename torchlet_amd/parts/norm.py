@@ -132,3 +132,40 @@ class ScalarRMSNorm(Norm):
         if rows is None:
             stream.pending = stream.post = stream.extra = None
         return out
+
+
+@NORMS.register("offset_rmsnorm")
+class OffsetRMSNorm(Norm):
+    """``r / sqrt(mean(r^2) + eps) * (offset + w) * gain`` with a weight vector ``w`` stored around zero (``offset`` 1), in 32-bit: the
+    offset and the fixed gain are folded into the vector once, at load, in 32-bit.  Like :class:`ScalarRMSNorm` it folds everything a
+    stream can carry (the pending branch output, normed with the weight its block left beside it; a second addend) in the same kernel."""
+    graph_safe = True
+    folds_post_norm = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.dim = spec.dim
+        self.eps = float(spec.eps)
+        self.weight: torch.Tensor | None = None
+
+    def weight_specs(self):
+        return {self.spec.weight_name: WeightSpec((self.dim,), keep=KEEP_FLOAT32, init="normal" if self.spec.offset else "one_plus_normal")}
+
+    def load_weights(self, tensors):
+        w = (tensors[self.spec.weight_name].to(torch.float32) + float(self.spec.offset)) * float(self.spec.gain)
+        self.weight = self._place(w, KEEP_FLOAT32)
+
+    def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0, read: torch.Tensor | None = None) -> torch.Tensor:
+        if stream.residual.dim() != 2 or stream.fold is not None:
+            raise ValueError("an offset_rmsnorm runs over one plain residual")
+        n = stream.residual.shape[0] if rows is None else rows.numel()
+        out = torch.empty((n, self.dim), dtype=self.dtype, device=stream.residual.device)
+        post_w, post_eps = stream.post if stream.post is not None else (None, 0.0)
+        ops.sandwich_norm(stream.residual, stream.pending, post_w, post_eps, stream.extra, self.weight, self.eps, out, rows, gain)
+        if rows is None:
+            stream.pending = stream.post = stream.extra = None
+        return out
+
+    def embed(self, token_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+        """``out[t] = norm(table[token_ids[t]] * scale)``: the embedding's rows normed on their way into the 32-bit stream, one kernel."""
+        ops.embedding_norm(token_ids, table, out, scale, self.weight, self.eps)

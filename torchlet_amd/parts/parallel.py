@@ -30,6 +30,8 @@ class ParallelMixer(Mixer):
         for name, b in zip(self.names, self.branches):
             if not isinstance(b, StagedMixer):
                 raise ConfigError(f"branch {name!r} of a parallel mixer is a {type(b).__name__}, which is not built in stages")
+        if any(getattr(b.spec, "qk_bias", False) or getattr(b.spec, "o_bias", False) for b in self.branches):
+            raise ConfigError("a parallel mixer stacks its branches' projections into one product; branches with biases are not built")
         if sum(b.paged_need() is not None for b in self.branches) > 1 or sum(b.state_need() is not None for b in self.branches) > 1:
             raise ConfigError("a parallel mixer holds one run's cache: at most one branch with pages and one with a state")
         self.hidden = spec.hidden

@@ -67,6 +67,18 @@ class PairRotaryEncoding(PositionEncoding):
             ops.rotate_pairs(flat, hd, 0, flat, hd, 0, positions, self.inv_freq, heads, hd)
 
 
+def scale_by_wavelength(freq: torch.Tensor, factor: float, low: float, high: float, original: float) -> torch.Tensor:
+    """Frequencies scaled band by band (64-bit): a frequency whose wavelength ``2 pi / f`` is shorter than ``original / high`` stays, one whose
+    wavelength is longer than ``original / low`` becomes ``f / factor``, and between the two ``(1 - s) f / factor + s f`` with ``s = (original /
+    wavelength - low) / (high - low)``."""
+    if not (factor > 0 and original > 0 and 0 < low < high):
+        raise ConfigError(f"rotary encoding: scaling by wavelength wants factor > 0, original > 0 and 0 < low < high, got {(factor, low, high, original)}")
+    wavelength = 2.0 * torch.pi / freq
+    s = (original / wavelength - low) / (high - low)
+    blended = (1.0 - s) * freq / factor + s * freq
+    return torch.where(wavelength < original / high, freq, torch.where(wavelength > original / low, freq / factor, blended))
+
+
 @POSITION_ENCODINGS.register("rope_halves")
 class HalfRotaryEncoding(PositionEncoding):
     """The rotate-half layout over the first ``dims`` entries of a vector: entry ``i`` is paired with ``i + dims / 2`` and the pair
@@ -84,7 +96,10 @@ class HalfRotaryEncoding(PositionEncoding):
         self.dims = spec.dims
         self.halves = True
         i = torch.arange(spec.dims // 2, dtype=torch.float64)
-        self.inv_freq = (float(spec.base) ** (-2.0 * i / spec.dims) / float(spec.factor)).to(torch.float32).to(device)
+        freq = float(spec.base) ** (-2.0 * i / spec.dims) / float(spec.factor)
+        if spec.bands is not None:
+            freq = scale_by_wavelength(freq, *(float(b) for b in spec.bands))
+        self.inv_freq = freq.to(torch.float32).to(device)
 
     def apply(self, q, k, positions):
         for x in (q, k):

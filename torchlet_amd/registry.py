@@ -9,6 +9,7 @@ import json
 from pathlib import Path
 
 from .config.base import ConfigError, ModelConfig
+from .config.bafulorn import BafulornConfig
 from .config.fotovik import FotovikConfig
 from .config.migurax import MiguraxConfig
 from .config.nebutar import NebutarConfig
@@ -32,6 +33,7 @@ register_architecture(Qwen2Config)
 register_architecture(MiguraxConfig)
 register_architecture(NebutarConfig)
 register_architecture(FotovikConfig)
+register_architecture(BafulornConfig)
 
 
 def config_class(name: str) -> type[ModelConfig]:
