@@ -48,6 +48,7 @@ def cpu_ops(monkeypatch):
                  "scaled_add_rmsnorm", "mlstm_scan", "gated_head_norm", "latent_tile_tokens", "latent_attention_mfma_fits", "latent_prepare", "rotate_pairs",
                  "latent_attention", "heads_linear", "experts_linear", "route", "combine", "activation", "compute_units",
                  "streams_norm", "delta_prepare", "delta_scan", "kv_cache_write", "local_attention", "local_attention_mfma_fits",
-                 "pool_blocks", "head_norm_rotate", "decay_scan", "silu_float", "bigram_embedding", "sandwich_norm", "normed_sum"):
+                 "pool_blocks", "head_norm_rotate", "decay_scan", "silu_float", "bigram_embedding", "sandwich_norm", "normed_sum",
+                 "selective_prepare", "selective_scan", "embedding_norm"):
         monkeypatch.setattr(ops, name, getattr(emulated_ops, name))
     return ops

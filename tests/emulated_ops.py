@@ -150,12 +150,19 @@ def interleave_gate_up(gate, up):
     return torch.stack((g.view(blocks, 32, K), u.view(blocks, 32, K)), dim=1).reshape(blocks * 64, K).contiguous()
 
 
-def linear_swiglu(x, gate_up, out):
+GATE_ACTIVATIONS = {"silu": 0, "relu": 1}
+
+
+def _gate(g, activation):
+    return torch.relu(g) if activation == "relu" else g / (1 + torch.exp(-g))
+
+
+def linear_swiglu(x, gate_up, out, activation="silu"):
     I, K = out.shape[1], x.shape[1]
     w = gate_up.float().view(-1, 2, 32, K)
     g = x.float() @ w[:, 0].reshape(-1, K)[:I].T
     u = x.float() @ w[:, 1].reshape(-1, K)[:I].T
-    out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
+    out.copy_((_gate(g, activation) * u).to(out.dtype))
 
 
 PREFILL_ATTENTION_ROWS = 64
@@ -185,10 +192,10 @@ def linear_partials(x, weight):
     return torch.stack((a, b))
 
 
-def swiglu(gate_up, out):
+def swiglu(gate_up, out, activation="silu"):
     I = gate_up.shape[1] // 2
     g, u = gate_up[:, :I].float(), gate_up[:, I:].float()
-    out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
+    out.copy_((_gate(g, activation) * u).to(out.dtype))
 
 
 def _mix32(x):
@@ -253,13 +260,53 @@ def mlstm_scan(qkv, k_off, v_off, gates, state, slots, req_indptr, out, heads, d
         st[:, dim * vdim + dim] = m
 
 
-def gated_head_norm(o, gate_values, weight, eps, out, heads, vdim, gate="sigmoid", gain=1.0):
+def gated_head_norm(o, gate_values, weight, eps, out, heads, vdim, gate="sigmoid", gain=1.0, gate_first=False):
     T = o.shape[0]
-    x = o.view(T, heads, vdim)
-    y = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight.float().view(-1, vdim)
     g = gate_values.float()
     g = torch.sigmoid(g) if gate == "sigmoid" else g * torch.sigmoid(g)
-    out.copy_((y.reshape(T, -1) * g * gain).to(out.dtype))
+    x = o.view(T, heads, vdim)
+    if gate_first:
+        x = x * g.reshape(T, heads, vdim)
+    y = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight.float().view(-1, vdim)
+    out.copy_((y.reshape(T, -1) * (1.0 if gate_first else g) * gain).to(out.dtype))
+
+
+def selective_prepare(proj, x_off, conv_w, conv_b, gates, a_log, dt_bias, state, tail_off, slots, req_indptr, token_req, qkv, heads, inner, gn, taps):
+    C = inner + 2 * gn
+    for r in range(req_indptr.numel() - 1):
+        lo, hi = int(req_indptr[r]), int(req_indptr[r + 1])
+        if hi <= lo:
+            continue
+        st = state[int(slots[r])]
+        tail = st[tail_off: tail_off + (taps - 1) * C].view(taps - 1, C)
+        x = torch.cat((tail, proj[lo:hi, x_off: x_off + C].float()), 0)
+        y = sum(x[j: j + hi - lo] * conv_w[:, j] for j in range(taps)) + conv_b
+        y = y * torch.sigmoid(y)
+        qkv[lo:hi] = torch.cat((y[:, inner + gn:], y[:, inner: inner + gn], y[:, :inner]), dim=1)          # C, B, x
+        if taps > 1:
+            tail.copy_(x[-(taps - 1):])
+    dt = torch.nn.functional.softplus(proj[:, x_off + C: x_off + C + heads].float() + dt_bias)
+    gates[:, :heads] = dt
+    gates[:, heads:] = torch.exp(-torch.exp(a_log) * dt)
+
+
+def selective_scan(qkv, gates, skip, state, slots, req_indptr, out, heads, groups, dim, vdim, max_new_tokens=None):
+    of = torch.arange(heads) // (heads // groups)
+    for r in range(req_indptr.numel() - 1):
+        st = state[int(slots[r])]
+        S = st[: heads * dim * vdim].view(heads, vdim, dim).transpose(1, 2).clone()
+        for t in range(int(req_indptr[r]), int(req_indptr[r + 1])):
+            q = qkv[t, : groups * dim].view(groups, dim)[of]
+            k = qkv[t, groups * dim: 2 * groups * dim].view(groups, dim)[of]
+            v = qkv[t, 2 * groups * dim:].view(heads, vdim)
+            S = S * gates[t, heads:, None, None] + k[:, :, None] * (gates[t, :heads, None] * v)[:, None, :]
+            out[t] = (torch.einsum("hde,hd->he", S, q) + skip[:, None] * v).reshape(-1)
+        st[: heads * dim * vdim] = S.transpose(1, 2).reshape(-1)
+
+
+def embedding_norm(token_ids, table, out, scale, weight, eps):
+    x = table.float()[token_ids.long()] * scale
+    out.copy_(x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight)
 
 
 DELTA_MAX_TAPS = 8
@@ -326,7 +373,7 @@ def local_attention_mfma_fits(dtype, dim, vdim, page_size):
 
 
 def local_attention(q, out, k_plane, v_plane, block_table, token_req, positions, heads, kv_heads, dim, vdim, page_size, scale,
-                    softcap=0.0, chunk=0, window=0, gain=1.0, tiles=None, sink=None, pooled=None):
+                    softcap=0.0, chunk=0, window=0, gain=1.0, tiles=None, sink=None, pooled=None, keep_first=0):
     group = heads // kv_heads
     for t in range(q.shape[0]):
         p, r = int(positions[t]), int(token_req[t])
@@ -335,7 +382,7 @@ def local_attention(q, out, k_plane, v_plane, block_table, token_req, positions,
             lo = max(lo, p // chunk * chunk)
         if window:
             lo = max(lo, p - window + 1)
-        keys = torch.arange(lo, p + 1)
+        keys = torch.cat((torch.arange(0, min(keep_first, lo)), torch.arange(lo, p + 1)))
         pages = block_table[r, keys // page_size].long()
         k = k_plane[pages, :, keys % page_size].float().repeat_interleave(group, dim=1)      # [n, heads, dim]
         v = v_plane[pages, :, :, keys % page_size].float().repeat_interleave(group, dim=1)
@@ -369,8 +416,10 @@ def pool_blocks(k_plane, v_plane, block_table, pk_plane, pv_plane, pool_table, r
             pv_plane[ppage, :, :, b % page_size] = v_plane[pages, :, :, keys % page_size].float().mean(0).to(pv_plane.dtype)
 
 
-def head_norm_rotate(x, heads_a, heads_b, dim, norm_a, norm_b, eps, positions, inv_freq, dims, halves):
+def head_norm_rotate(x, heads_a, heads_b, dim, norm_a, norm_b, eps, positions, inv_freq, dims, halves, raw_b=None):
     T = x.shape[0]
+    if raw_b is not None:
+        raw_b.copy_(x[:, heads_a * dim:])
     v = x.float().reshape(T, heads_a + heads_b, dim).clone()
     if norm_a is not None or norm_b is not None:
         w = torch.cat([(norm_a if norm_a is not None else torch.ones(dim)).float().expand(heads_a, dim),
@@ -479,15 +528,16 @@ def _turn(x, positions, inv_freq):
     return y
 
 
-def latent_prepare(down, q_rank, rank, rot, rot_dims, wq, wkv, eps, positions, inv_freq, cq, token_req=None, block_table=None,
+def latent_prepare(down, q_rank, kv_off, rank, rot, rot_dims, wq, wkv, eps, positions, inv_freq, cq, token_req=None, block_table=None,
                    plane=None, page_size=0):
     x = down.float()
     norm = lambda t, w: t / torch.sqrt(t.pow(2).mean(-1, keepdim=True) + eps) * w.float()
-    cq.copy_(norm(x[:, :q_rank], wq).to(cq.dtype))
+    if q_rank:
+        cq.copy_(norm(x[:, :q_rank], wq).to(cq.dtype))
     if plane is None:
         return
-    c = norm(x[:, q_rank: q_rank + rank], wkv)
-    kr = _turn(x[:, q_rank + rank: q_rank + rank + rot], positions, inv_freq)
+    c = norm(x[:, kv_off: kv_off + rank], wkv)
+    kr = _turn(x[:, kv_off + rank: kv_off + rank + rot], positions, inv_freq)
     row = torch.cat((c, kr), dim=-1).to(plane.dtype)
     for t in range(down.shape[0]):
         p = int(positions[t])
@@ -505,7 +555,7 @@ def rotate_pairs(src, src_head, src_off, dst, dst_head, dst_off, positions, inv_
 
 
 def latent_attention(q, out, plane, block_table, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles, tile_tokens, heads, rank, rot,
-                     page_size, scale, sink, splits=1, general=False, max_new_tokens=None):
+                     page_size, scale, sink, splits=1, general=False, max_new_tokens=None, window=0, gate=None):
     D = rank + rot
     for tile in range(num_tiles):
         if tile_req is None:
@@ -516,7 +566,7 @@ def latent_attention(q, out, plane, block_table, req_indptr, ctx_lens, tile_req,
         ctx = int(ctx_lens[r])
         for i in range(t0, min(t0 + tile_tokens, n_new)):
             pos = ctx + i
-            keys = torch.arange(0, pos + 1)
+            keys = torch.arange(max(0, pos - window + 1) if window else 0, pos + 1)
             rows = plane[block_table[r, keys // page_size].long(), 0, keys % page_size].float()     # [n, D]
             s = (q[first + i].float().view(heads, D) @ rows.T) * scale
             top = s.max(-1, keepdim=True).values
@@ -524,7 +574,10 @@ def latent_attention(q, out, plane, block_table, req_indptr, ctx_lens, tile_req,
                 top = torch.maximum(top, sink[:, None])
             e = torch.exp(s - top)
             den = e.sum(-1, keepdim=True) + (torch.exp(sink[:, None] - top) if sink is not None else 0.0)
-            out[first + i] = ((e / den) @ rows[:, :rank]).reshape(-1).to(out.dtype)
+            o = (e / den) @ rows[:, :rank]
+            if gate is not None:
+                o = o * torch.sigmoid(gate[first + i, :heads].float())[:, None]
+            out[first + i] = o.reshape(-1).to(out.dtype)
 
 
 def heads_linear(x, x_head, weight, out, out_head, general=False):
@@ -555,15 +608,21 @@ def experts_linear(x, slot_token, weight, offsets, out, activation="none", gener
             out[lo:hi] = _act(rows.float() @ weight[e].float().T, activation).to(out.dtype)
 
 
-def route(logits, top, scores="chosen", choice_bias=None):
+def route(logits, top, scores="chosen", choice_bias=None, weight_scale=1.0, weight_eps=0.0):
     T, E = logits.shape
     if scores == "all":
         s = torch.softmax(logits, dim=-1)
         best = (s if choice_bias is None else s + choice_bias).topk(top, dim=-1)
         weights = s.gather(1, best.indices)
+    elif scores == "sigmoid":
+        s = torch.sigmoid(logits)
+        best = (s if choice_bias is None else s + choice_bias).topk(top, dim=-1)
+        weights = s.gather(1, best.indices)
+        weights = weights / (weights.sum(-1, keepdim=True) + weight_eps)
     else:
         best = logits.topk(top, dim=-1)               # ties: not met in tests
         weights = torch.softmax(best.values, dim=-1)
+    weights = weights * weight_scale
     chosen = best.indices.reshape(-1)
     order = torch.sort(chosen, stable=True).indices
     slot_token = (order // top).to(torch.int32)
@@ -574,14 +633,17 @@ def route(logits, top, scores="chosen", choice_bias=None):
     return weights, offsets, slot_token, pair_slot
 
 
-def combine(y, pair_slot, weights, out, identity=None):
+def combine(y, pair_slot, weights, out, identity=None, addend=None):
     T, top = weights.shape
     rows = y[pair_slot.long()].float().view(T, top, -1)
     if identity is not None:
         x, offsets, experts = identity
         own = (pair_slot >= offsets[experts]).view(T, top, 1)
         rows = torch.where(own, x.float()[:, None, :], rows)
-    out.copy_((rows * weights[:, :, None]).sum(1).to(out.dtype))
+    total = (rows * weights[:, :, None]).sum(1)
+    if addend is not None:
+        total = total + addend.float()
+    out.copy_(total.to(out.dtype))
 
 
 def activation(x, kind):

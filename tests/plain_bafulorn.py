@@ -7,8 +7,9 @@ head; grouped-query attention whose values are its unrotated keys, with a partia
 keeps the first tokens; a selective state-space recurrence behind a short convolution); feed-forwards that are dense and gated (relu) or
 routed over gated experts (silu) by a sigmoid router with a shared expert; a final norm and a head.
 
-``forward(config, tensors, tokens, stored=None)`` returns ``(logits [T, vocab], the stream after every layer)``.  ``stored``: a function
-applied to every tensor that separate kernels hand to each other in the engine (the yardstick of the bfloat16 engine's rounding).
+``forward(config, tensors, tokens, stored=None, gaps=None)`` returns ``(logits [T, vocab], the stream after every layer)``.  ``stored``: a
+function applied to every tensor that separate kernels hand to each other in the engine (the yardstick of the bfloat16 engine's
+rounding).  ``gaps``: a list that receives every router's margin of choice, token by token.
 """
 from __future__ import annotations
 
@@ -181,18 +182,22 @@ def gated_ff(h, w, prefix, act, stored=_same):
     return stored(act(h @ w[prefix + "gate"].T) * (h @ w[prefix + "up"].T)) @ w[prefix + "down"].T
 
 
-def sigmoid_router(h, w, router: dict):
+def sigmoid_router(h, w, router: dict, gaps=None):
     """Scores ``s = sigmoid(W_r h)``; the ``top`` largest of ``s + correction`` are chosen (the lower index wins a tie); their weights are
-    ``s / (sum of the chosen s + 1e-20) * scale``.  Returns ``(chosen [T, top], weights [T, top])``."""
+    ``s / (sum of the chosen s + 1e-20) * scale``.  Returns ``(chosen [T, top], weights [T, top])``.  ``gaps``: a list that receives, per
+    token, by how much the last chosen expert's choice score leads the best one left out."""
     s = torch.sigmoid(h @ w["router"].T)
     choice = s + w["correction"]
-    chosen = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, : router["top"]]
+    ranked = torch.sort(choice, dim=-1, descending=True, stable=True)
+    chosen = ranked.indices[:, : router["top"]]
+    if gaps is not None and router["top"] < choice.shape[1]:
+        gaps.extend((ranked.values[:, router["top"] - 1] - ranked.values[:, router["top"]]).tolist())
     picked = torch.gather(s, 1, chosen)
     return chosen, picked / (picked.sum(-1, keepdim=True) + 1e-20) * router["scale"]
 
 
-def routed_ff(h, w, mlp, stored=_same):
-    chosen, weights = sigmoid_router(h, w, mlp["router"])
+def routed_ff(h, w, mlp, stored=_same, gaps=None):
+    chosen, weights = sigmoid_router(h, w, {"scale": 1.0, **mlp["router"]}, gaps)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for j in range(chosen.shape[1]):
@@ -209,8 +214,8 @@ def under(tensors, prefix):
     return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
 
 
-def forward(config, tensors, tokens, stored=_same):
-    eps, m = float(config["norm"]["eps"]), float(config["residual_mult"])
+def forward(config, tensors, tokens, stored=_same, gaps=None):
+    eps, m = float(config["norm"]["eps"]), float(config.get("residual_mult", 1.0))
     x = offset_rms_norm(tensors["embed"][torch.as_tensor(tokens)], tensors["embed.norm"], eps)
     after = []
     for i, layer in enumerate(config["layers"]):
@@ -230,7 +235,7 @@ def forward(config, tensors, tokens, stored=_same):
         if mlp is not None:
             h = stored(offset_rms_norm(x, w["norm2"], eps))
             ff = under(w, "mlp.")
-            y = gated_ff(h, ff, "", torch.relu, stored) if mlp["kind"] == "dense" else routed_ff(h, ff, mlp, stored)
+            y = gated_ff(h, ff, "", torch.relu, stored) if mlp["kind"] == "dense" else routed_ff(h, ff, mlp, stored, gaps)
             x = x + m * offset_rms_norm(stored(y), w["norm2b"], eps)
         after.append(x.clone())
     h = stored(offset_rms_norm(x, tensors["final.norm"], eps))
