@@ -174,7 +174,8 @@ latent_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, 
     const int* table = block_table + (size_t)req * bt_stride;
     // with a window a row at qpos reads the keys qpos - window + 1 .. qpos; the tile starts at the step of LAT_KT keys (counted from
     // position 0, so that a key's step does not depend on the tile) in which its first row's first key lies
-    const int kbegin = window > 0 ? max(0, ctx + tok0 - window + 1) / LAT_KT * LAT_KT : 0;
+    const int tile_first = window > 0 ? max(0, ctx + tok0 - window + 1) : 0;
+    const int kbegin = tile_first / LAT_KT * LAT_KT;
     const int qfirst = window > 0 ? max(0, qpos - window + 1) : 0;
     for (int k0 = kbegin + split * LAT_KT; k0 <= last; k0 += splits * LAT_KT) {
         __syncthreads();
@@ -182,7 +183,8 @@ latent_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, 
         for (int i = threadIdx.x; i < nk * D; i += blockDim.x) {
             const int kk = i / D, d = i % D, pos = k0 + kk;
             const int page = table[pos / page_size];
-            sk[kk * ldk + d] = to_float(plane[((size_t)page * page_size + pos % page_size) * D + d]);
+            // (what lies before the tile's first key may be gone with its page: it counts as zeros)
+            sk[kk * ldk + d] = pos >= tile_first ? to_float(plane[((size_t)page * page_size + pos % page_size) * D + d]) : 0.f;
         }
         __syncthreads();
         if (!row_ok || k0 > qpos || k0 + nk <= qfirst) continue;
@@ -327,6 +329,7 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
     const int rt = row_ok ? row / hchunk : 0, rh = head0 + (row_ok ? row % hchunk : 0);
     const int tok = first + tok0 + rt, qpos = ctx + tok0 + rt;
     const int qfirst = window > 0 ? max(0, qpos - window + 1) : 0;      // the first key this query reads
+    const int tile_first = window > 0 ? max(0, ctx + tok0 - window + 1) : 0;      // ... and the first one any query of the tile reads
     LmFrag qf[LM_DC_MAX];
 #pragma unroll
     for (int c = 0; c < LM_DC_MAX; ++c)
@@ -366,7 +369,7 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
     // (every lane fetches, from a clamped place where its own lies beyond the keys or the row: a fetch under a condition
     // would be waited for on the spot; what must be zero is cleared when the pieces are written to shared memory)
     auto request = [&](uint4 (&stage)[LM_DC_MAX / 2], int at) {
-        const int pos = min(at + kk, last);
+        const int pos = max(min(at + kk, last), tile_first);
         const int blk = page_shift >= 0 ? pos >> page_shift : pos / page_size;
         const bf16_t* src = plane + ((size_t)tbl[blk] * page_size + (pos - blk * page_size)) * D;
 #pragma unroll
@@ -379,7 +382,7 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
         for (int i = 0; i < LM_DC_MAX / 2; ++i) {
             if (i < rounds) {
                 const int col = 64 * i + 8 * pg;
-                const uint4 x = (k0 + kk <= last && col < D) ? stage[i] : make_uint4(0, 0, 0, 0);
+                const uint4 x = (k0 + kk <= last && k0 + kk >= tile_first && col < D) ? stage[i] : make_uint4(0, 0, 0, 0);
                 // the neighbour's half: the even lane keeps its first four numbers and gets the neighbour's, the odd lane the last four
                 const uint32_t mine0 = odd ? x.z : x.x, mine1 = odd ? x.w : x.y;
                 const uint32_t got0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)(odd ? x.x : x.z), 0xB1, 0xF, 0xF, true);
@@ -470,7 +473,7 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
         }
     };
     // (with a window the tile starts at the step, counted from position 0, in which its first token's first key lies)
-    const int kfirst = (window > 0 ? max(0, ctx + tok0 - window + 1) / LM_KEYS * LM_KEYS : 0) + split * LM_KEYS;
+    const int kfirst = tile_first / LM_KEYS * LM_KEYS + split * LM_KEYS;
     if (kfirst <= last) request(stage0, kfirst);
     if constexpr (TWO) {
         if (kfirst + stride <= last) request(stage1, kfirst + stride);

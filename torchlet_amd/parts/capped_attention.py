@@ -87,10 +87,10 @@ class CappedAttention(StagedMixer):
         return ["local_attention"]
 
     def weight_specs(self):
-        specs = {"q": WeightSpec((self.q_width, self.hidden)), "k": WeightSpec((self.k_width, self.hidden)),
-                 "o": WeightSpec((self.hidden, self.mix_width))}
+        specs = {"q": WeightSpec((self.q_width, self.hidden)), "k": WeightSpec((self.k_width, self.hidden))}
         if not self.shared_kv:
             specs["v"] = WeightSpec((self.v_width, self.hidden))
+        specs["o"] = WeightSpec((self.hidden, self.mix_width))
         if self.spec.qk_bias:
             specs["q.b"] = WeightSpec((self.q_width,), keep=KEEP_STORED)
             specs["k.b"] = WeightSpec((self.k_width,), keep=KEEP_STORED)

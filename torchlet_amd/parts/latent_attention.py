@@ -72,16 +72,18 @@ class LatentAttention(Mixer):
 
     def weight_specs(self):
         H, n = self.hidden, self.heads
-        specs = {
-            "dkv": WeightSpec((self.row, H)), "dkv.norm": WeightSpec((self.rank,), keep=KEEP_STORED, init="one_plus_normal"),
-            "uk": WeightSpec((n * self.dim, self.rank)), "uv": WeightSpec((n * self.vdim, self.rank)),
-            "o": WeightSpec((H, n * self.vdim)),
-        }
+        # (the order of declaration is the order of the random-weights mode's draws)
+        specs = {}
         if self.q_rank:
             specs.update({"dq": WeightSpec((self.q_rank, H)), "dq.norm": WeightSpec((self.q_rank,), keep=KEEP_STORED, init="one_plus_normal"),
                           "uq": WeightSpec((n * (self.dim + self.rot), self.q_rank))})
         else:
             specs["q"] = WeightSpec((n * (self.dim + self.rot), H))
+        specs.update({
+            "dkv": WeightSpec((self.row, H)), "dkv.norm": WeightSpec((self.rank,), keep=KEEP_STORED, init="one_plus_normal"),
+            "uk": WeightSpec((n * self.dim, self.rank)), "uv": WeightSpec((n * self.vdim, self.rank)),
+            "o": WeightSpec((H, n * self.vdim)),
+        })
         if self.spec.sink:
             specs["sink"] = WeightSpec((n,), keep=KEEP_FLOAT32)
         if self.spec.gate:
