@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16]
                     [--shape 7b|14b|32b] [--context N] [--new-tokens G] [--prefill-tokens T]
-                    [--workload decode|serve|migurax|nebutar|fotovik] [--only decode|step|prefill] [--all]
+                    [--workload decode|serve|migurax|nebutar|fotovik|bafulorn] [--only decode|step|prefill] [--all]
 
 The default run has the layer sizes of Qwen2.5-7B (28 layers, hidden 3584, 28 heads, 4 KV heads, head
 size 128, intermediate 18944, vocabulary 152064) with random weights and goes through the whole engine
@@ -49,6 +49,12 @@ kernels beside the like kernels of the Migurax and Qwen2 paths.
 pooled blocks before it and a sink; causal attention with normed queries and keys beside linear attention with fixed decays; a gated
 delta rule; dense feed-forwards), beside the Nebutar model of the same width and layer count (the closest one the framework has: two
 mixers side by side, a delta rule, a span of layers, the same attention kernels), and its own kernels beside their like.
+
+``--workload bafulorn [--size s|m]`` does the same for the Bafulorn design (a norm before and after every sublayer with weights around zero;
+attention over a cached latent in a window with a gate; grouped-query attention whose values are its keys, in a window that keeps the
+first tokens; a selective state-space recurrence; gated dense feed-forwards and experts routed by sigmoid scores with a shared expert),
+beside the Migurax model of the same width and layer count (the closest one the framework has: latent attention, a recurrent state per
+request, routed experts), and the kernels it added or changed beside their like.
 """
 from __future__ import annotations
 
@@ -91,8 +97,8 @@ def parse_args(argv=None):
     p.add_argument("--context", type=int, default=CONTEXT, help="prompt tokens of each request in the decode runs")
     p.add_argument("--new-tokens", type=int, default=None, help="tokens each request may generate (decode: 256, serve: 128)")
     p.add_argument("--prefill-tokens", type=int, default=2048)
-    p.add_argument("--workload", choices=["decode", "serve", "migurax", "nebutar", "fotovik"], default="decode")
-    p.add_argument("--size", choices=["s", "m"], default="s", help="migurax, nebutar, fotovik: layer sizes (s: width 2048, m: width 4096)")
+    p.add_argument("--workload", choices=["decode", "serve", "migurax", "nebutar", "fotovik", "bafulorn"], default="decode")
+    p.add_argument("--size", choices=["s", "m"], default="s", help="migurax, nebutar, fotovik, bafulorn: layer sizes (s: width 2048, m: width 4096)")
     p.add_argument("--requests", type=int, default=32)
     p.add_argument("--prompt-min", type=int, default=128)
     p.add_argument("--prompt-max", type=int, default=4096)
@@ -1086,6 +1092,222 @@ def fotovik(args) -> dict:
     return out
 
 
+# ---------------------------------------------------------------------------------------------- the Bafulorn design
+
+def bafulorn_sizes(size: str) -> dict:
+    """A Bafulorn configuration of four layers at the width of the other designs' sizes: attention over a latent of 512 numbers with heads
+    of 128 in a window of 1024 with a gate, with experts; grouped-query attention with heads of 128 whose values are its keys, half a head
+    rotated with scaled frequencies, in a window of 1024 that keeps the first four tokens, with a gated dense feed-forward; a selective
+    state-space recurrence with heads of 64 over twice the width, states of 128 numbers, a convolution of four taps, with experts; and the
+    latent attention once more with a dense feed-forward."""
+    width, heads, ff, experts, eff, top = dict(s=(2048, 16, 5632, 16, 1024, 2), m=(4096, 32, 11264, 32, 2048, 4))[size]
+    latent = dict(heads=heads, dim=128, vdim=128, kv_rank=512, scale=128 ** -0.5, mask=dict(size=1024))
+    attention = dict(heads=heads, kv_heads=heads // 4, dim=128, vdim=128, scale=128 ** -0.5, mask=dict(size=1024, keep_first=4),
+                     rot=dict(dims=64, base=500000.0, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
+    mamba = dict(heads=2 * width // 64, vdim=64, state=128, groups=1, conv=4, norm_groups=1)
+    moe = dict(kind="moe", expert=dict(ff=eff), router=dict(experts=experts, top=top, scale=2.5), shared=dict(ff=eff))
+    dense = dict(kind="dense", ff=ff)
+    return dict(architecture="Bafulorn", vocab=32000, width=width, max_positions=8192, norm=dict(eps=1e-6), residual_mult=0.3,
+                layers=[dict(type="latent_attention", mixer=latent, mlp=moe), dict(type="attention", mixer=attention, mlp=dense),
+                        dict(type="mamba2", mixer=mamba, mlp=moe), dict(type="latent_attention", mixer=latent, mlp=dense)])
+
+
+def bafulorn_kernels(ours: dict, like: dict, batch: int, context: int, tokens: int) -> list[dict]:
+    """Each kernel that the design added or changed, alone, at the sizes of ``ours``, in a decode step of ``batch`` requests on ``context`` cached
+    tokens and in a prompt of ``tokens`` tokens, beside the like kernel of the closest path the framework had.  ``frac``: bytes that must
+    move / time against 8 TB/s, or operations / time against the matrix cores' bfloat16 rate (against the 32-bit rate for the recurrence)."""
+    import torch
+    from torchlet_amd.kernels import ops
+    dev, bf = "cuda", torch.bfloat16
+    rows = []
+
+    def add(name, kind, launch, nbytes=0.0, flops=0.0, peak=MFMA_PEAK_TFLOPS["bfloat16"]):
+        ms = _best_ms(launch, rounds=3, calls=5)
+        row = {"kernel": name, "like": kind, "ms": round(ms, 4)}
+        if nbytes:
+            row.update(bytes=int(nbytes), frac=round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), bound="hbm")
+        else:
+            row.update(flops=flops, frac=round(flops / (ms * 1e-3) / (peak * 1e12), 4), bound="flops")
+        rows.append(row)
+        say(f"  {name}: {ms:.4f} ms, {row['frac']} of its bound")
+
+    def tables(n_req, total):
+        blocks = -(-total // PAGE)
+        table = (torch.arange(n_req * blocks, dtype=torch.int32, device=dev) + 1).view(n_req, blocks)
+        return table, n_req * blocks + 1
+
+    width = ours["width"]
+    lat, att, ssm = ours["layers"][0]["mixer"], ours["layers"][1]["mixer"], ours["layers"][2]["mixer"]
+    moe = ours["layers"][0]["mlp"]
+    # ---- the selective recurrence beside the delta rule (the same kernel with its correction): a decode step reads and writes every
+    #      state once; a prompt does 4 operations per state element and token (the update and one sum over the rows), the delta rule 6
+    h, p_, n_, g_ = ssm["heads"], ssm["vdim"], ssm["state"], ssm["groups"]
+    inner, gn = h * p_, g_ * n_
+    for name, T, reqs in (("selective_scan decode", batch, batch), (f"selective_scan prompt {tokens}", tokens, 1)):
+        cbx = torch.randn(T, 2 * gn + inner, device=dev) * 0.1
+        gates = torch.rand(T, 2 * h, device=dev) * 0.5 + 0.5
+        skip = torch.ones(h, device=dev)
+        state = torch.zeros(reqs + 1, h * n_ * p_ + 3 * (inner + 2 * gn), device=dev)
+        out = torch.empty(T, inner, device=dev)
+        slots = torch.arange(reqs, dtype=torch.int32, device=dev)
+        indptr = (torch.arange(reqs + 1, dtype=torch.int32, device=dev) * (T // reqs))
+        launch = lambda: ops.selective_scan(cbx, gates, skip, state, slots, indptr, out, h, g_, n_, p_, max_new_tokens=T // reqs)
+        dh, dg, dd, dv_ = h, max(1, h // 2), n_, p_              # a delta rule with states of the same size
+        qkv2 = torch.randn(T, 2 * dg * dd + dh * dv_, device=dev) * 0.1
+        out2 = torch.empty(T, dh * dv_, device=dev)
+        launch2 = lambda: ops.delta_scan(qkv2, gates, state, slots, indptr, out2, dh, dg, dd, dv_, max_new_tokens=T // reqs)
+        if reqs > 1:
+            add(name, "delta_scan decode", launch, nbytes=2.0 * reqs * h * n_ * p_ * 4)
+            add("delta_scan decode (states of the same size)", "", launch2, nbytes=2.0 * reqs * h * n_ * p_ * 4)
+        else:
+            add(name, f"delta_scan prompt {tokens}", launch, flops=4.0 * T * h * n_ * p_, peak=MFMA_PEAK_TFLOPS["float32"])
+            add(f"delta_scan prompt {tokens} (states of the same size)", "", launch2, flops=6.0 * T * h * n_ * p_, peak=MFMA_PEAK_TFLOPS["float32"])
+    # ---- what the recurrence reads (convolution with its bias, silu, step sizes and decays) beside the delta rule's: the projection read, the
+    #      32-bit channels written
+    T = tokens
+    C = inner + 2 * gn
+    proj = (torch.randn(T, 2 * inner + 2 * gn + h, device=dev) * 0.3).to(bf)
+    conv_w, conv_b = torch.randn(C, 4, device=dev) * 0.3, torch.zeros(C, device=dev)
+    gates, cbx = torch.empty(T, 2 * h, device=dev), torch.empty(T, C, device=dev)
+    a_log, dt_bias = torch.zeros(h, device=dev), torch.zeros(h, device=dev)
+    state = torch.zeros(2, h * n_ * p_ + 3 * C, device=dev)
+    one_req = (torch.zeros(1, dtype=torch.int32, device=dev), torch.tensor([0, T], dtype=torch.int32, device=dev), torch.zeros(T, dtype=torch.int32, device=dev))
+    add(f"selective_prepare prompt {tokens}", "delta_prepare", lambda: ops.selective_prepare(proj, inner, conv_w, conv_b, gates, a_log, dt_bias, state, h * n_ * p_, *one_req,
+                                                                                              cbx, h, inner, gn, 4), nbytes=float(T) * C * 6)
+    dgates, dqkv = torch.randn(T, 2 * h, device=dev), torch.empty(T, C, device=dev)         # a delta rule with as many channels: 2 kv_heads x state + heads x vdim
+    if gn % n_ == 0 and n_ <= 256 and p_ <= 256:
+        add(f"delta_prepare prompt {tokens} (as many channels)", "", lambda: ops.delta_prepare(proj, conv_w, dgates, a_log, dt_bias, state, h * n_ * p_, *one_req, dqkv, h, g_, n_, p_, 4,
+                                                                                             1.0, 1e-6), nbytes=float(T) * C * 6)
+    y, z = torch.randn(T, inner, device=dev), (torch.randn(T, inner, device=dev)).to(bf)
+    wn, outn = torch.ones(inner, device=dev), torch.empty(T, inner, dtype=bf, device=dev)
+    add(f"gated_head_norm prompt {tokens}, gate before the norm, one group", "gated_head_norm", lambda: ops.gated_head_norm(y, z, wn, 1e-6, outn, 1, inner, gate="silu", gate_first=True),
+        nbytes=float(T) * inner * 8)
+    add(f"gated_head_norm prompt {tokens}, per head of {p_} (delta rule's)", "", lambda: ops.gated_head_norm(y, z, wn, 1e-6, outn, h, p_, gate="silu"), nbytes=float(T) * inner * 8)
+    # ---- attention over the cached latent in a window with a gate, beside the causal one with a sink (the Migurax path): a decode step reads the
+    #      rows it may see once; a prompt's scores and sums over the latent
+    H, rank = lat["heads"], lat["kv_rank"]
+    for label, window, gated, sink_on in ((f"window {lat['mask']['size']}, gate", lat["mask"]["size"], True, False), ("causal, sink (Migurax path)", 0, False, True)):
+        for T, reqs, ctx in ((batch, batch, context - 1), (tokens, 1, 0)):
+            total = ctx + T // reqs
+            table, pages = tables(reqs, total)
+            plane = (torch.randn(pages, 1, PAGE, rank, device=dev) * 0.3).to(bf)
+            q = (torch.randn(T, H * rank, device=dev) * 0.1).to(bf)
+            out = torch.empty(T, H * rank, dtype=bf, device=dev)
+            gate = (torch.randn(T, H, device=dev)).to(bf) if gated else None
+            sink = torch.zeros(H, device=dev) if sink_on else None
+            tq = ops.latent_tile_tokens(H, ops.LATENT_MFMA_ROWS)
+            keys = min(total, window + T // reqs - 1) if window else total
+            if reqs == 1:
+                n_tiles = -(-T // tq)
+                args = (torch.tensor([0, T], dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int32, device=dev), torch.zeros(n_tiles, dtype=torch.int32, device=dev),
+                        torch.arange(n_tiles, dtype=torch.int32, device=dev) * tq, n_tiles)
+                splits = 1
+            else:
+                args = (None, torch.full((reqs,), ctx, dtype=torch.int32, device=dev), None, None, reqs)
+                splits = max(1, min(256 // reqs, keys // 64, 64))
+            launch = lambda: ops.latent_attention(q, out, plane, table, *args, tq, H, rank, 0, PAGE, 0.09, sink, splits, max_new_tokens=T // reqs, window=window, gate=gate)
+            seen = lambda p: min(p + 1, window) if window else p + 1
+            if reqs > 1:
+                add(f"latent_attention decode, {label}", "latent_attention decode, causal", launch, nbytes=float(reqs) * seen(ctx) * rank * 2)
+            else:
+                add(f"latent_attention prompt {tokens}, {label}", f"latent_attention prompt {tokens}, causal", launch, flops=4.0 * H * rank * sum(seen(p) for p in range(T)))
+    # ---- attention in a window that keeps the first tokens, beside the plain window (the same kernels): a decode step reads the keys and values
+    #      it may see once; a prompt's scores and sums
+    H, G, dk = att["heads"], att["kv_heads"], att["dim"]
+    for label, keep in ((f"window {att['mask']['size']}, {att['mask']['keep_first']} kept", att["mask"]["keep_first"]), ("plain window", 0)):
+        window = att["mask"]["size"]
+        for T, reqs, ctx in ((batch, batch, context - 1), (tokens, 1, 0)):
+            total = ctx + T // reqs
+            table, pages = tables(reqs, total)
+            k_plane = (torch.randn(pages, G, PAGE, dk, device=dev) * 0.3).to(bf)
+            v_plane = (torch.randn(pages, G, dk, PAGE, device=dev) * 0.3).to(bf)
+            q = (torch.randn(T, H * dk, device=dev) * 0.3).to(bf)
+            out = torch.empty(T, H * dk, dtype=bf, device=dev)
+            token_req = torch.arange(T, dtype=torch.int32, device=dev) // (T // reqs)
+            positions = (torch.arange(T, dtype=torch.int32, device=dev) % (T // reqs)) + ctx
+            if reqs == 1:
+                n_tiles = -(-T // ops.LOCAL_ATTENTION_TILE_TOKENS)
+                tiles = (torch.tensor([0, T], dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int32, device=dev),
+                         torch.zeros(n_tiles, dtype=torch.int32, device=dev), torch.arange(n_tiles, dtype=torch.int32, device=dev) * ops.LOCAL_ATTENTION_TILE_TOKENS, n_tiles)
+            else:
+                tiles = (torch.arange(reqs + 1, dtype=torch.int32, device=dev), torch.full((reqs,), ctx, dtype=torch.int32, device=dev), None, None, reqs)
+            launch = lambda: ops.local_attention(q, out, k_plane, v_plane, table, token_req, positions, H, G, dk, dk, PAGE, att["scale"], 0.0, 0, window, 1.0,
+                                                 tiles=tiles, keep_first=keep)
+            seen = lambda p: min(p + 1, window) + min(keep, max(0, p - window + 1))
+            if reqs > 1:
+                add(f"local_attention decode, {label}", "local_attention decode, plain window", launch, nbytes=float(reqs) * seen(ctx) * G * 2 * dk * 2)
+            else:
+                add(f"local_attention prompt {tokens}, {label}", f"local_attention prompt {tokens}, plain window", launch, flops=4.0 * H * dk * sum(seen(p) for p in range(T)))
+    # ---- the rotation with the keys copied as they come, beside the rotation alone; the norm with a weight vector beside the plain residual's
+    #      norm; the embedding with its norm beside the embedding; the sigmoid router beside the softmax one
+    T = tokens
+    x = torch.randn(T, (H + G) * dk, device=dev).to(bf)
+    raw = torch.empty(T, G * dk, dtype=bf, device=dev)
+    positions = torch.arange(T, dtype=torch.int32, device=dev)
+    inv = torch.rand(att["rot"]["dims"] // 2, device=dev)
+    add(f"head_norm_rotate prompt {tokens}, keys copied", "head_norm_rotate", lambda: ops.head_norm_rotate(x, H, G, dk, None, None, 0.0, positions, inv, att["rot"]["dims"], True, raw_b=raw),
+        nbytes=float(T) * ((H + G) * dk * 4 + G * dk * 2))
+    add(f"head_norm_rotate prompt {tokens} (Fotovik path)", "", lambda: ops.head_norm_rotate(x, H, G, dk, None, None, 0.0, positions, inv, att["rot"]["dims"], True),
+        nbytes=float(T) * (H + G) * dk * 4)
+    for name, T in (("sandwich_norm decode, weight vectors", batch), (f"sandwich_norm prompt {tokens}, weight vectors", tokens)):
+        res = torch.randn(T, width, device=dev)
+        pen = torch.randn(T, width, device=dev).to(bf)
+        wv = torch.ones(width, device=dev)
+        out = torch.empty(T, width, dtype=bf, device=dev)
+        add(name, "add_rmsnorm", lambda: ops.sandwich_norm(res, pen, wv, 1e-6, None, wv, 1e-6, out), nbytes=float(T) * width * 12)
+        wb = torch.ones(width, dtype=bf, device=dev)
+        add(name.split(",")[0].replace("sandwich_norm", "add_rmsnorm") + " (Qwen2 path)", "", lambda: ops.add_rmsnorm(res, pen, wb, 1e-5, out), nbytes=float(T) * width * 12)
+    T = tokens
+    emb = torch.randn(ours["vocab"], width, device=dev).to(bf)
+    ids = torch.randint(0, ours["vocab"], (T,), dtype=torch.int32, device=dev)
+    res2, wv = torch.empty(T, width, device=dev), torch.ones(width, device=dev)
+    add(f"embedding_norm prompt {tokens}", "embedding", lambda: ops.embedding_norm(ids, emb, res2, 1.0, wv, 1e-6), nbytes=float(T) * width * 6)
+    add(f"embedding prompt {tokens} (Qwen2 path)", "", lambda: ops.embedding(ids, emb, res2, 1.0), nbytes=float(T) * width * 6)
+    E, top = moe["router"]["experts"], moe["router"]["top"]
+    logits, corr = torch.randn(T, E, device=dev), torch.zeros(E, device=dev)
+    add(f"route prompt {tokens}, sigmoid scores", "route", lambda: ops.route(logits, top, "sigmoid", corr, 2.5, 1e-20), nbytes=float(T) * (E * 4 + top * 16))
+    add(f"route prompt {tokens}, softmax over all (Nebutar path)", "", lambda: ops.route(logits, top, "all", corr), nbytes=float(T) * (E * 4 + top * 16))
+    # ---- the gated feed-forward's first product with relu in its epilogue beside silu (the Qwen2 path's kernel)
+    ff = ours["layers"][1]["mlp"]["ff"]
+    gate_up = ops.interleave_gate_up((torch.randn(ff, width, device=dev) * 0.02).to(bf), (torch.randn(ff, width, device=dev) * 0.02).to(bf))
+    for T in (batch, tokens):
+        xx = torch.randn(T, width, device=dev).to(bf)
+        zz = torch.empty(T, ff, dtype=bf, device=dev)
+        kind = "decode" if T == batch else f"prompt {tokens}"
+        if T == batch:
+            add(f"linear_swiglu {kind}, relu", "linear_swiglu", lambda: ops.linear_swiglu(xx, gate_up, zz, "relu"), nbytes=2.0 * ff * width * 2)
+            add(f"linear_swiglu {kind}, silu (Qwen2 path)", "", lambda: ops.linear_swiglu(xx, gate_up, zz, "silu"), nbytes=2.0 * ff * width * 2)
+        else:
+            add(f"linear_swiglu {kind}, relu", "linear_swiglu", lambda: ops.linear_swiglu(xx, gate_up, zz, "relu"), flops=4.0 * T * ff * width)
+            add(f"linear_swiglu {kind}, silu (Qwen2 path)", "", lambda: ops.linear_swiglu(xx, gate_up, zz, "silu"), flops=4.0 * T * ff * width)
+    return rows
+
+
+def bafulorn(args) -> dict:
+    import torch
+    ours = bafulorn_sizes(args.size)
+    like = migurax_sizes(args.size)[0]
+    out = {"metric": f"Bafulorn design, size {args.size} (width {ours['width']}, 4 layers), prefill of {args.prefill_tokens} tokens and decode at batch "
+                     f"{args.batch} on {args.context}-token caches, beside the Migurax design at equal width and layer count, one MI355X",
+           "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+           "data": "synthetic: seeded random weights, token ids and cache contents", "config": {"bafulorn": ours, "migurax": like}}
+    for key, d in (("bafulorn", ours), ("migurax", like)):
+        say(f"building the {key} model")
+        cfg, model = _build_from(d, args.dtype)
+        pms, pbest = time_prefill(model, args.prefill_tokens)
+        dms = _decode_ms(model, args.batch, min(args.steps, 64), args.warmup, args.context)
+        out[key] = {"weight_bytes": _weight_bytes(model),
+                    "prefill": {"tokens": args.prefill_tokens, "ms": round(pms, 3), "ms_best": round(pbest, 3), "tokens_per_s": round(args.prefill_tokens * 1e3 / pms, 1)},
+                    "decode": {"batch": args.batch, "context": args.context, "ms_per_step": round(dms, 4), "tokens_per_s": round(args.batch * 1e3 / dms, 1)}}
+        say(f"{key}: {out[key]}")
+        del model
+        torch.cuda.empty_cache()
+    out["value"] = out["bafulorn"]["decode"]["tokens_per_s"]
+    if args.dtype == "bfloat16" and not args.no_points:
+        out["kernels"] = bafulorn_kernels(ours, like, args.batch, args.context, args.prefill_tokens)
+    return out
+
+
 def main(argv=None) -> int:
     args = parse_args(argv)
     args.serve_new_tokens = args.new_tokens or 128
@@ -1105,6 +1327,9 @@ def main(argv=None) -> int:
         return 0
     if args.workload == "fotovik":
         print(json.dumps(fotovik(args)))
+        return 0
+    if args.workload == "bafulorn":
+        print(json.dumps(bafulorn(args)))
         return 0
     name, sizes = SHAPES[args.shape]
     full_layers = sizes["num_hidden_layers"]

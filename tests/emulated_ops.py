@@ -528,8 +528,9 @@ def _turn(x, positions, inv_freq):
     return y
 
 
-def latent_prepare(down, q_rank, kv_off, rank, rot, rot_dims, wq, wkv, eps, positions, inv_freq, cq, token_req=None, block_table=None,
-                   plane=None, page_size=0):
+def latent_prepare(down, q_rank, rank, rot, rot_dims, wq, wkv, eps, positions, inv_freq, cq, token_req=None, block_table=None,
+                   plane=None, page_size=0, kv_off=None):
+    kv_off = q_rank if kv_off is None else kv_off
     x = down.float()
     norm = lambda t, w: t / torch.sqrt(t.pow(2).mean(-1, keepdim=True) + eps) * w.float()
     if q_rank:

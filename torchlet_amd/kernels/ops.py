@@ -1295,13 +1295,15 @@ def latent_attention_mfma_fits(dtype: torch.dtype, heads: int, rank: int, rot: i
     return dtype == torch.bfloat16 and bool(_lib("latent").tl_latent_attention_mfma_fits(c_int(rank), c_int(rot), c_int(heads * (rank + rot))))
 
 
-def latent_prepare(down: torch.Tensor, q_rank: int, kv_off: int, rank: int, rot: int, rot_dims: int, wq: torch.Tensor | None, wkv: torch.Tensor,
+def latent_prepare(down: torch.Tensor, q_rank: int, rank: int, rot: int, rot_dims: int, wq: torch.Tensor | None, wkv: torch.Tensor,
                    eps: float, positions: torch.Tensor, inv_freq: torch.Tensor, cq: torch.Tensor | None, token_req: torch.Tensor | None = None,
-                   block_table: torch.Tensor | None = None, plane: torch.Tensor | None = None, page_size: int = 0) -> None:
+                   block_table: torch.Tensor | None = None, plane: torch.Tensor | None = None, page_size: int = 0, kv_off: int | None = None) -> None:
     """From the fused first projection ``down [T, >= kv_off + rank + rot]``: ``cq = rmsnorm(down[:, :q_rank]) * wq`` (``q_rank`` 0: no query
     latent, ``wq`` and ``cq`` ``None``) and, with a plane ``[pages, 1, page, rank + rot]``, the token's cache row ``[rmsnorm(down[:, kv_off:kv_off +
-    rank]) * wkv, the next rot numbers with the first rot_dims of them turned in pairs by the token's position]``."""
+    rank]) * wkv, the next rot numbers with the first rot_dims of them turned in pairs by the token's position]``.  ``kv_off``: the column
+    where the key/value latent starts (default: right after the query latent)."""
     T = down.shape[0]
+    kv_off = q_rank if kv_off is None else kv_off
     if down.stride(1) != 1 or kv_off < q_rank or down.shape[1] < kv_off + rank + rot or (q_rank == 0) != (cq is None) or (q_rank == 0) != (wq is None) \
             or (cq is not None and (cq.shape != (T, q_rank) or cq.dtype != down.dtype or not cq.is_contiguous())):
         raise KernelError("latent_prepare: shapes do not fit")

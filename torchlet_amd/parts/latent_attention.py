@@ -122,13 +122,13 @@ class LatentAttention(Mixer):
         write = (ctx.token_req, table, plane, cache.page_size) if cache.writable else (None, None, None, 0)
         if self.q_rank:
             cq = torch.empty((T, self.q_rank), dtype=self.dtype, device=dev)
-            ops.latent_prepare(down, self.q_rank, self.q_cols, self.rank, self.rot, rot_dims, self.w_dq_norm, self.w_dkv_norm, float(self.spec.norm_eps),
+            ops.latent_prepare(down, self.q_rank, self.rank, self.rot, rot_dims, self.w_dq_norm, self.w_dkv_norm, float(self.spec.norm_eps),
                                ctx.positions, inv_freq, cq, *write)
             q = torch.empty((T, n * (self.dim + self.rot)), dtype=self.dtype, device=dev)
             ops.linear(cq, self.w_uq, None, q)
         else:                       # the queries are the first columns of the projection
-            ops.latent_prepare(down, 0, self.q_cols, self.rank, self.rot, rot_dims, None, self.w_dkv_norm, float(self.spec.norm_eps),
-                               ctx.positions, inv_freq, None, *write)
+            ops.latent_prepare(down, 0, self.rank, self.rot, rot_dims, None, self.w_dkv_norm, float(self.spec.norm_eps),
+                               ctx.positions, inv_freq, None, *write, kv_off=self.q_cols)
             q = down[:, : self.q_cols]
         # the query against a cache row: [W_uk^T q_unrotated, rotated part], head by head
         qrow = torch.empty((T, n * self.row), dtype=self.dtype, device=dev)
