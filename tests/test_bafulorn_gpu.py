@@ -188,6 +188,37 @@ def test_configurations_drawn_at_random(tmp_path, seed):
             assert runner.cache.live_requests() == [] and runner.cache.free_pages() == runner.cache.capacity()
 
 
+MIDDLE = dict(architecture="Bafulorn", vocab=1000, width=256, norm=dict(eps=1e-6), residual_mult=0.35, layers=[
+    dict(type="latent_attention", mixer=dict(heads=8, dim=64, vdim=48, kv_rank=256, scale=0.125, mask=dict(size=96)),
+         mlp=dict(kind="moe", expert=dict(ff=128), router=dict(experts=8, top=2, scale=2.0), shared=dict(ff=192))),
+    dict(type="attention", mixer=dict(heads=8, kv_heads=2, dim=128, vdim=128, scale=0.09, mask=dict(size=70, keep_first=9),
+                                      rot=dict(dims=64, base=100000.0, scaling=dict(factor=8.0, low=1.0, high=4.0, original=256))),
+         mlp=dict(kind="dense", ff=640)),
+    dict(type="mamba2", mixer=dict(heads=16, vdim=32, state=64, groups=2, conv=4, norm_groups=4), mlp=dict(kind="dense", ff=512)),
+    dict(type="attention", mixer=dict(heads=6, kv_heads=6, dim=96, vdim=96, scale=0.1, mask=dict(size=33, keep_first=2), rot=dict(dims=96, base=10000.0)),
+         mlp=dict(kind="moe", expert=dict(ff=96), router=dict(experts=5, top=3, scale=1.5))),
+    dict(type="mamba2", mixer=dict(heads=6, vdim=64, state=128, groups=1, conv=3, norm_groups=1), mlp=None),
+    dict(type="latent_attention", mixer=dict(heads=20, dim=32, vdim=64, kv_rank=128, scale=0.18, mask=dict(size=40)), mlp=dict(kind="dense", ff=384)),
+])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sizes_between_the_tiny_ones_and_a_real_model(tmp_path, dtype):
+    """Widths and heads at which the products run on their tile kernels and the attentions in whole tiles: whole requests, portions and
+    mixed batches against the plain implementation."""
+    from torchlet_amd.engine.loading import load_model, make_runner
+    folder = tiny_bafulorn.write("middle", tmp_path, config=MIDDLE, seed=51)
+    w = {k: v.double() for k, v in tiny_bafulorn.tensors_for("middle", 1.0, MIDDLE, 51).items()}
+    seqs, refs = tiny_bafulorn.sequences("", w, [230, 3, 121, 64], seed=3, config=MIDDLE, min_gap=0.02)
+    tol = dict(atol=8e-4, rtol=3e-4) if dtype == "float32" else _bf16_bound(MIDDLE, w, seqs, refs)
+    _, model = load_model(folder, dtype)
+    for mode in ("whole", "portions", "mixed"):
+        steps = scenarios.number(getattr(scenarios, mode)(seqs))
+        runner = make_runner(model, page_size=16, num_pages=-(-scenarios.max_tokens_needed(steps, unit=16) // 16) + 1, max_requests=4)
+        scenarios.check(steps, _replay(runner, steps), refs, tol, f"middle/{mode}/{dtype}")
+        assert runner.cache.live_requests() == [] and runner.cache.free_pages() == runner.cache.capacity()
+
+
 SHARP = dict(architecture="Bafulorn", vocab=80, width=64, norm=dict(eps=1e-5), residual_mult=0.5, layers=[
     dict(type="attention", mixer=dict(heads=4, kv_heads=1, dim=32, vdim=32, scale=0.3, rot=dict(dims=8, base=10000.0), mask=dict(size=32, keep_first=5)),
          mlp=dict(kind="dense", ff=64)),
