@@ -1105,9 +1105,9 @@ def bafulorn_sizes(size: str) -> dict:
     attention = dict(heads=heads, kv_heads=heads // 4, dim=128, vdim=128, scale=128 ** -0.5, mask=dict(size=1024, keep_first=4),
                      rot=dict(dims=64, base=500000.0, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
     mamba = dict(heads=2 * width // 64, vdim=64, state=128, groups=1, conv=4, norm_groups=1)
-    moe = dict(kind="moe", expert=dict(ff=eff), router=dict(experts=experts, top=top, scale=2.5), shared=dict(ff=eff))
+    moe = dict(kind="moe", expert=dict(ff=eff), router=dict(experts=experts, top=top, scale=2.0), shared=dict(ff=eff))
     dense = dict(kind="dense", ff=ff)
-    return dict(architecture="Bafulorn", vocab=32000, width=width, max_positions=8192, norm=dict(eps=1e-6), residual_mult=0.3,
+    return dict(architecture="Bafulorn", vocab=32000, width=width, max_positions=8192, norm=dict(eps=1e-6), residual_mult=0.25,
                 layers=[dict(type="latent_attention", mixer=latent, mlp=moe), dict(type="attention", mixer=attention, mlp=dense),
                         dict(type="mamba2", mixer=mamba, mlp=moe), dict(type="latent_attention", mixer=latent, mlp=dense)])
 
@@ -1265,7 +1265,7 @@ def bafulorn_kernels(ours: dict, like: dict, batch: int, context: int, tokens: i
     add(f"embedding prompt {tokens} (Qwen2 path)", "", lambda: ops.embedding(ids, emb, res2, 1.0), nbytes=float(T) * width * 6)
     E, top = moe["router"]["experts"], moe["router"]["top"]
     logits, corr = torch.randn(T, E, device=dev), torch.zeros(E, device=dev)
-    add(f"route prompt {tokens}, sigmoid scores", "route", lambda: ops.route(logits, top, "sigmoid", corr, 2.5, 1e-20), nbytes=float(T) * (E * 4 + top * 16))
+    add(f"route prompt {tokens}, sigmoid scores", "route", lambda: ops.route(logits, top, "sigmoid", corr, 2.0, 1e-20), nbytes=float(T) * (E * 4 + top * 16))
     add(f"route prompt {tokens}, softmax over all (Nebutar path)", "", lambda: ops.route(logits, top, "all", corr), nbytes=float(T) * (E * 4 + top * 16))
     # ---- the gated feed-forward's first product with relu in its epilogue beside silu (the Qwen2 path's kernel)
     ff = ours["layers"][1]["mlp"]["ff"]

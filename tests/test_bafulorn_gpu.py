@@ -189,7 +189,7 @@ def test_configurations_drawn_at_random(tmp_path, seed):
 
 
 MIDDLE = dict(architecture="Bafulorn", vocab=1000, width=256, norm=dict(eps=1e-6), residual_mult=0.35, layers=[
-    dict(type="latent_attention", mixer=dict(heads=8, dim=64, vdim=48, kv_rank=256, scale=0.125, mask=dict(size=96)),
+    dict(type="latent_attention", mixer=dict(heads=8, dim=96, vdim=48, kv_rank=256, scale=0.1, mask=dict(size=100)),
          mlp=dict(kind="moe", expert=dict(ff=128), router=dict(experts=8, top=2, scale=2.0), shared=dict(ff=192))),
     dict(type="attention", mixer=dict(heads=8, kv_heads=2, dim=128, vdim=128, scale=0.09, mask=dict(size=70, keep_first=9),
                                       rot=dict(dims=64, base=100000.0, scaling=dict(factor=8.0, low=1.0, high=4.0, original=256))),

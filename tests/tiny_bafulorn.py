@@ -62,8 +62,8 @@ CONFIGS = {
         dict(type="mamba2", mixer=_mamba(3, 7, 9, 1, 4, 1), mlp=_moe(8, 4, 3, 0.8)),
     ]),
     # sizes of the matrix-core kernels, pages of 16; windows that are no multiples of the page; kept tokens that span two pages
-    "B": dict(architecture="Bafulorn", vocab=80, width=64, norm=dict(eps=3e-6), residual_mult=0.3, layers=[
-        dict(type="latent_attention", mixer=_latent(4, 32, 48, 64, 0.18, window=40), mlp=_moe(32, 6, 3, 2.5, 32)),
+    "B": dict(architecture="Bafulorn", vocab=80, width=64, norm=dict(eps=3e-6), residual_mult=0.25, layers=[
+        dict(type="latent_attention", mixer=_latent(4, 32, 48, 64, 0.18, window=40), mlp=_moe(32, 6, 3, 2.2, 32)),
         dict(type="attention", mixer=_attention(4, 2, 64, 0.12, rot=_rot(32, 50000.0, (8.0, 1.0, 4.0, 512)), window=24, keep_first=20), mlp=_dense(96)),
         dict(type="mamba2", mixer=_mamba(4, 32, 32, 2, 4, 2), mlp=_dense(64)),
         dict(type="latent_attention", mixer=_latent(2, 64, 32, 128, 0.125, window=21), mlp=None),
@@ -203,7 +203,7 @@ def random_config(rnd, big: bool) -> dict:
         else:
             experts = rnd.choice([2, 4, 7])
             mlp = _moe(rnd.choice([8, 24, 32]), experts, rnd.choice([1, 2, 3, experts]) if experts > 2 else rnd.choice([1, 2]),
-                       rnd.choice([None, 1.0, 2.5]), rnd.choice([None, 16, 40]))
+                       rnd.choice([None, 1.0, 2.2]), rnd.choice([None, 16, 40]))
         layers.append(dict(type=kind, mixer=mixer, mlp=mlp))
     return dict(architecture="Bafulorn", vocab=rnd.choice([31, 90, 300]), width=rnd.choice([64, 128] if big else [24, 40, 56]),
                 norm=dict(eps=rnd.choice([1e-5, 1e-6, 3e-4])), residual_mult=rnd.choice([1.0, 0.3, 0.55]), layers=layers)

@@ -324,6 +324,38 @@ __global__ void gated_head_norm_kernel(const float* __restrict__ o, const T* __r
     }
 }
 
+// The same for long stretches (more than 512 numbers normed together: all heads of a mixer as one): a work-group of 256 threads per token and
+// stretch instead of a wave, the sum of squares joined through shared memory.
+template <typename T>
+__global__ void __launch_bounds__(256)
+gated_row_norm_kernel(const float* __restrict__ o, const T* __restrict__ gate, int gate_ld, const void* __restrict__ weight, int weight_f32,
+                      int shared_weight, float eps, T* __restrict__ out, int out_ld, int heads, int vdim, int gate_kind, float gain, int gate_first) {
+    __shared__ float red[16];
+    const int row = blockIdx.x;
+    const int t = row / heads, h = row % heads;
+    const float* src = o + (size_t)row * vdim;
+    const T* g = gate + (size_t)t * gate_ld + h * vdim;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < vdim; i += blockDim.x) {
+        float u = src[i];
+        if (gate_first) {
+            const float z = to_float(g[i]);
+            const float s = 1.f / (1.f + expf(-z));
+            u *= gate_kind == 1 ? z * s : s;
+        }
+        ss = fmaf(u, u, ss);
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float)vdim + eps);
+    T* dst = out + (size_t)t * out_ld + h * vdim;
+    const int w0 = shared_weight ? 0 : h * vdim;
+    for (int i = threadIdx.x; i < vdim; i += blockDim.x) {
+        const float z = to_float(g[i]);
+        const float s = 1.f / (1.f + expf(-z));
+        dst[i] = from_float<T>(src[i] * (gate_kind == 1 ? z * s : s) * inv * load_vec(weight, weight_f32, w0 + i) * gain);
+    }
+}
+
 extern "C" int tl_gated_head_norm(const void* o, const void* gate, int gate_ld, const void* weight, int weight_f32, int shared_weight, float eps,
                                   void* out, int out_ld, int tokens, int heads, int vdim, int gate_kind, float gain, int gate_first, int dtype,
                                   hipStream_t stream) {
@@ -331,6 +363,17 @@ extern "C" int tl_gated_head_norm(const void* o, const void* gate, int gate_ld, 
     TL_REQUIRE(gate_kind == 0 || gate_kind == 1, "gated_head_norm: unknown gate %d", gate_kind);
     if (tokens == 0) return TL_OK;
     const int rows = tokens * heads;
+    if (vdim > 512) {
+        if (dtype == TL_DT_F32)
+            gated_row_norm_kernel<float><<<rows, 256, 0, stream>>>((const float*)o, (const float*)gate, gate_ld, weight, weight_f32, shared_weight, eps,
+                                                                   (float*)out, out_ld, heads, vdim, gate_kind, gain, gate_first);
+        else if (dtype == TL_DT_BF16)
+            gated_row_norm_kernel<bf16_t><<<rows, 256, 0, stream>>>((const float*)o, (const bf16_t*)gate, gate_ld, weight, weight_f32, shared_weight, eps,
+                                                                    (bf16_t*)out, out_ld, heads, vdim, gate_kind, gain, gate_first);
+        else TL_REQUIRE(false, "gated_head_norm: unknown dtype %d", dtype);
+        TL_CHECK_LAUNCH("gated_row_norm");
+        return TL_OK;
+    }
     dim3 grid((rows + 3) / 4), block(4 * TL_WAVE);
     if (dtype == TL_DT_F32)
         gated_head_norm_kernel<float><<<grid, block, 0, stream>>>((const float*)o, (const float*)gate, gate_ld, weight, weight_f32, shared_weight, eps,
