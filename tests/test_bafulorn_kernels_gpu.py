@@ -293,7 +293,10 @@ def test_latent_attention_with_a_window_and_a_gate(dtype, H, rank, page, window)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_latent_rows_at_the_window_edge_carry_the_weight_or_none(dtype):
+@pytest.mark.parametrize("decoded", [False, True])
+def test_latent_rows_at_the_window_edge_carry_the_weight_or_none(dtype, decoded):
+    """One query at the end of 300 tokens (in a portion, or decoded alone) whose first head matches one cached row: at the first position of
+    the window and at a page border inside it the row comes through whole; just outside the window, and far back, it does not show at all."""
     H, rank, page, window, n = 2, 64, 16, 40, 300
     last = n - 1
     g = torch.Generator().manual_seed(8)
@@ -302,7 +305,7 @@ def test_latent_rows_at_the_window_edge_carry_the_weight_or_none(dtype):
         q, c = torch.randn(n, H * rank, generator=g) * 0.2, torch.randn(n, rank, generator=g) * 0.2
         c[at] = torch.randn(rank, generator=g)
         q[last, :rank] = c[at] * 3.0
-        _, _, _, outs, fits = _latent_attend(dtype, H, rank, page, window, [n], [[150, 290]], g, scale=1.0, q=[q], c=[c], gated=False)
+        _, _, _, outs, fits = _latent_attend(dtype, H, rank, page, window, [n], [[n - 1]] if decoded else [[150, 290]], g, scale=1.0, q=[q], c=[c], gated=False)
         want = _plain_latent(q, c, None, H, rank, window, dtype, scale=1.0, gated=False)[last]
         for use_mfma in ((False, True) if fits else (False,)):
             got = outs[use_mfma][0][last].double()
