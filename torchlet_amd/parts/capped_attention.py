@@ -123,8 +123,7 @@ class CappedAttention(StagedMixer):
         v_plane = v_plane.view(v_plane.shape[0], self.kv_heads, self.vdim, cache.page_size)
         table = ctx.block_tables[cache.group]
         q = proj[:, : self.q_width]
-        values = None
-        if self.shared_kv:          # the keys as projected, copied before they are normed and turned
+        if self.shared_kv:          # the keys as projected: the kernel that turns them copies them here first
             values = torch.empty((proj.shape[0], self.k_width), dtype=self.dtype, device=proj.device)
         else:
             values = proj[:, self.q_width + self.k_width:]
